@@ -4,5 +4,7 @@ from .base import ConfigError, ConfigReader, LayerKinds, architecture_name, read
 from .qwen3 import Qwen3Config
 from .gokazen import GokazenConfig
 from .pudorax import PudoraxConfig
+from .dupidra import DupidraConfig
 
-__all__ = ["ConfigError", "ConfigReader", "architecture_name", "read_config_json", "LayerKinds", "Qwen3Config", "GokazenConfig", "PudoraxConfig"]
+__all__ = ["ConfigError", "ConfigReader", "architecture_name", "read_config_json", "LayerKinds", "Qwen3Config", "GokazenConfig", "PudoraxConfig",
+           "DupidraConfig"]

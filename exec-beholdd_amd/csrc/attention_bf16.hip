@@ -172,7 +172,7 @@ __global__ __launch_bounds__(256, (LEAN ? 2 : 1)) void attention_mfma_kernel(
   const int pos_row = positions[row];                   // the row's own position
   const bool new_key_apart = FUSED && fused.write_kv;   // the key at pos_row is not in the cache yet
   const int pos = new_key_apart ? pos_row - 1 : pos_row;   // the last key the row takes from the cache (-1: none)
-  const int lo = (window > 0 && pos_row - window + 1 > 0) ? pos_row - window + 1 : 0;
+  const int lo = bh_first_visible(pos_row, window);
   bf16x8_t q_vec[NS];
   // FUSED: the raw rows and what norms and rotates them are asked for here and used once the first page's
   // loads are under way (q) and after the pages (the new key and value).
@@ -514,7 +514,7 @@ static int attention_bf16_run(const void* q, void* out, void* part_o, void* part
   BH_REQUIRE(n_seqs > 0 && n_rows > 0 && max_rows_per_seq > 0, "attention_bf16: empty batch");
   BH_REQUIRE(H > 0 && KVH > 0 && H % KVH == 0, "attention_bf16: %d query heads do not group evenly into %d kv heads", H, KVH);
   BH_REQUIRE(hd % 32 == 0 && hd >= 32 && hd <= 256, "attention_bf16: head size %d is not a multiple of 32 up to 256", hd);
-  BH_REQUIRE(window >= 0 && max_position >= 0, "attention_bf16: window and positions must not be negative");
+  BH_REQUIRE(max_position >= 0, "attention_bf16: positions must not be negative");
   BH_REQUIRE(n_splits >= 1 && (n_splits == 1 || (part_o && part_ml)), "attention_bf16: split keys need scratch memory");
   const int G = H / KVH;
   const int tiles = (max_rows_per_seq * G + 15) / 16;

@@ -92,7 +92,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NS <= 4 ? 2
   const int group_last_col = min(n_cols, group_col0 + GROUP_TILES * 16) - 1;
   const int group_pos_max = positions[row0 + group_last_col / G];
   const int group_pos_first = positions[row0 + group_col0 / G];
-  const int group_lo_min = (window > 0 && group_pos_first - window + 1 > 0) ? group_pos_first - window + 1 : 0;
+  const int group_lo_min = bh_first_visible(group_pos_first, window);
   const int begin = group_lo_min / BH_PAGE, last = group_pos_max / BH_PAGE;
   const int32_t* table = page_table + (size_t)seq * table_stride;
 
@@ -108,7 +108,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NS <= 4 ? 2
     const int c = wanted < n_cols ? wanted : n_cols - 1;
     const int row = row0 + c / G, head = kvh * G + c % G;
     pos[ct] = positions[row];
-    lo[ct] = (window > 0 && pos[ct] - window + 1 > 0) ? pos[ct] - window + 1 : 0;
+    lo[ct] = bh_first_visible(pos[ct], window);
     pos_max = max(pos_max, pos[ct]);
     pos_min = min(pos_min, pos[ct]);
     lo_min = min(lo_min, lo[ct]);

@@ -730,7 +730,7 @@ extern "C" int bh_qk_norm_rope_cache_sums(const float* sums, int parts, void* q_
 
 // ---- attention over the paged cache, any size -------------------------------------------------
 // One block per (row, query head).  The row at position p of sequence s sees keys
-// max(0, p - window + 1) .. p of that sequence (window 0: all of them).  Keys are taken 256
+// bh_first_visible(p, window) .. p of that sequence (a window, a chunk or all of them: csrc/layout.h).  Keys are taken 256
 // at a time: scores (one thread per key), running maximum and sum in float32 (online softmax),
 // then the value sum with threads spread over (key subset, dimension).
 
@@ -751,7 +751,7 @@ __global__ __launch_bounds__(THREADS) void attention_generic_kernel(
   const int kv_head = head / (H / KVH);
   const int pos = positions[row];
   const int32_t* table = page_table + (size_t)row_seq[row] * table_stride;
-  const int first = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int first = bh_first_visible(pos, window);
 
   const T* qr = q + ((size_t)row * H + head) * hd;
   for (int i = tid; i < hd; i += THREADS) qs[i] = to_f32(qr[i]);
@@ -811,7 +811,6 @@ extern "C" int bh_attention_generic(const void* q, void* out, int dtype, const v
   BH_REQUIRE(H % KVH == 0, "attention: %d query heads do not group evenly into %d kv heads", H, KVH);
   BH_REQUIRE(hd <= 1024, "attention: head size %d is above the limit of 1024", hd);
   BH_REQUIRE(H <= 65535, "attention: too many heads");
-  BH_REQUIRE(window >= 0, "attention: window must not be negative");
   BH_REQUIRE(kv_order == BH_KV_ROWS || (kv_order == BH_KV_PIECES && hd % 32 == 0),
              "attention: cache order %d does not exist for head size %d", kv_order, hd);
   const int threads = hd <= AG_THREADS ? AG_THREADS : (hd <= 512 ? 512 : 1024);

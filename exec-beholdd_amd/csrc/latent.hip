@@ -85,7 +85,7 @@ extern "C" int bh_latent_write(const void* down, int dtype, int row_stride, int 
   BH_REQUIRE(query == nullptr || (H > 0 && q_first >= 0 && src_first >= 0 && q_first + rot_dim <= q_head && src_first + rot_dim <= src_head &&
                                   (long)H * q_head <= q_row && H * src_head <= row_stride),
              "latent_write: the heads' rotated slices do not lie inside their rows");
-  BH_REQUIRE(n_rows > 0 && rank > 0 && rot_dim > 0, "latent_write: sizes must be positive");
+  BH_REQUIRE(n_rows > 0 && rank > 0 && rot_dim >= 0, "latent_write: sizes must be positive (the rotated part may be absent)");
   BH_REQUIRE(turned >= 0 && turned % 2 == 0 && turned <= rot_dim, "latent_write: %d turned dimensions of %d", turned, rot_dim);
   BH_REQUIRE(turned == 0 || freq != nullptr, "latent_write: a rotation needs its frequencies");
   BH_REQUIRE(offset >= 0 && offset + rank + rot_dim <= row_stride, "latent_write: the latent does not lie inside a row of %d", row_stride);

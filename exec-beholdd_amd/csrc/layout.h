@@ -41,6 +41,17 @@ BH_BOTH inline int bh_value_index(int order, int token, int dim, int hd) {
   return (((dt * 2 + u) * 64) + 16 * g + j) * 8 + token % 8;
 }
 
+// ---- which keys a query sees ------------------------------------------------------------------
+// The attention kernels take one number, `span`, for how far back a query at position p looks: 0 for every key up
+// to its own, w > 0 for a window (the last w positions, its own among them), -c < 0 for chunks of c positions
+// counted from the sequence's position 0 (the keys of the query's own chunk up to its own position).  The first key
+// seen never moves back as p grows, which is all that the kernels' page walks assume.
+BH_BOTH inline int bh_first_visible(int position, int span) {
+  if (span > 0) return position - span + 1 > 0 ? position - span + 1 : 0;
+  if (span < 0) return position - position % (-span);
+  return 0;
+}
+
 // ---- activation rows in blocks ---------------------------------------------------------------
 // A bfloat16 matrix [rows][width] that a product of many rows reads as its activations may be kept in
 // blocks of 16 rows x 32 columns, each 1 KB in the order in which one matrix-core operand lies in a

@@ -1,0 +1,242 @@
+// A matrix memory with exponential gates (mLSTM), walked as a recurrence over a float32 state.  Per sequence and head:
+//   i_t = cap tanh(x_i / cap),  f_t = logsigmoid(cap tanh(x_f / cap))        the gates' logarithms, from their pre-activations
+//   m_t = max(f_t + m_(t-1), i_t)                                            m starts at 0
+//   a_t = exp(f_t + m_(t-1) - m_t),  b_t = exp(i_t - m_t)
+//   S_t = a_t S_(t-1) + b_t k_t v_t^T,   n_t = a_t n_(t-1) + b_t k_t           S [dim][vdim], n [dim], zero at the start
+//   o_t = S_t^T q_t / (max(|n_t . q_t|, exp(-m_t)) + 1e-6)
+// n is S's column for a value that is always one, so the state of a head is kept as vdim + 1 columns of dim floats (the
+// last one n), then m: (vdim + 1) * dim + 1 floats a head, heads one after the other in a slot's row of the cache.
+//   mlstm_gates    a_t, b_t and m_t of every row and head, the rows of a sequence in order from the slot's m, which it moves on
+//   mlstm_scan     the recurrence over the columns: S^T q and n . q of every row and head, from the slot's state, which it moves on
+//   mlstm_finish   the division, the heads' RMS norm (no mean taken off), the weight and the sigmoid gate, for the output projection
+// Everything here is float32 but the projected q, k, v and the gate's pre-activation, which come in the activation type.
+#include "common.h"
+
+#define ML_BESIDE 4      // floats a row and head beside the read-out: a_t, b_t, m_t, n_t . q_t
+
+// ---- the gates -------------------------------------------------------------------------------------------------
+// A wave a (sequence, head).  64 rows at a time: every lane makes its row's two logarithms, then all lanes walk the 64
+// steps of m together (a step needs the one before), each keeping its own row's.
+__global__ __launch_bounds__(BH_WAVE) void mlstm_gates_kernel(const float* __restrict__ pre, const float* __restrict__ bias, float cap,
+                                                              float* __restrict__ state, long slot_stride, int head_floats,
+                                                              const int32_t* __restrict__ seq_start, const int32_t* __restrict__ seq_slot,
+                                                              float* __restrict__ beside, int H) {
+  const int seq = blockIdx.x / H, head = blockIdx.x % H, lane = threadIdx.x;
+  const int row0 = seq_start[seq], rows = seq_start[seq + 1] - row0;
+  float* m_at = state + (size_t)seq_slot[seq] * slot_stride + (size_t)head * head_floats + head_floats - 1;
+  float m = *m_at;
+  const float bias_i = bias ? bias[head] : 0.f, bias_f = bias ? bias[H + head] : 0.f, inv_cap = 1.0f / cap;
+  for (int base = 0; base < rows; base += BH_WAVE) {
+    const int t = base + lane;
+    float gate_i = 0.f, gate_f = 0.f;
+    if (t < rows) {
+      const float* x = pre + (size_t)(row0 + t) * 2 * H;
+      gate_i = cap * tanhf((x[head] + bias_i) * inv_cap);
+      const float z = cap * tanhf((x[H + head] + bias_f) * inv_cap);
+      gate_f = fminf(z, 0.f) - log1pf(expf(-fabsf(z)));      // log(sigmoid(z)) without overflow
+    }
+    float before = 0.f, mine = 0.f;
+    const int steps = rows - base < BH_WAVE ? rows - base : BH_WAVE;
+    for (int s = 0; s < steps; ++s) {
+      const float f_s = __shfl(gate_f, s, BH_WAVE), i_s = __shfl(gate_i, s, BH_WAVE);
+      const float next = fmaxf(f_s + m, i_s);
+      if (s == lane) {
+        before = m;
+        mine = next;
+      }
+      m = next;
+    }
+    if (t < rows) {
+      float* out = beside + ((size_t)(row0 + t) * H + head) * ML_BESIDE;
+      out[0] = expf(gate_f + before - mine);
+      out[1] = expf(gate_i - mine);
+      out[2] = mine;
+    }
+  }
+  if (lane == 0 && rows > 0) *m_at = m;
+}
+
+// pre f32 [n_rows][2 H]: the input gates' pre-activations of the H heads, then the forget gates'; bias f32 [2 H] or null.
+extern "C" int bh_mlstm_gates(const float* pre, const float* bias, float cap, float* state, long slot_stride, int head_floats,
+                              const int32_t* seq_start, const int32_t* seq_slot, float* beside, int n_seqs, int H, hipStream_t stream) {
+  BH_REQUIRE(n_seqs > 0 && H > 0 && head_floats > 0 && cap > 0.f, "mlstm_gates: sizes and the cap must be positive");
+  BH_REQUIRE((long)H * head_floats <= slot_stride, "mlstm_gates: %d heads of %d floats do not fit a slot's %ld", H, head_floats, slot_stride);
+  mlstm_gates_kernel<<<n_seqs * H, BH_WAVE, 0, stream>>>(pre, bias, cap, state, slot_stride, head_floats, seq_start, seq_slot, beside, H);
+  return bh_check_launch("mlstm_gates");
+}
+
+// ---- the recurrence --------------------------------------------------------------------------------------------
+// A workgroup a (sequence, head, tile of 16 columns).  Thread (column c, slice s) keeps rows s, s + 16, ... of column c in
+// registers; the 16 slices of a column are neighbouring lanes, so a row's read-out is added up inside the wave.  16 rows of q, k,
+// the tile's values and the gates' factors go through LDS at a time, the next 16 asked for before these are walked.
+#define ML_COLS 16
+#define ML_SLICES 16
+#define ML_STAGE 16
+
+template <typename T, int R>
+__global__ __launch_bounds__(ML_COLS * ML_SLICES) void mlstm_scan_kernel(
+    const T* __restrict__ proj, int row_stride, int q_off, int k_off, int v_off, const float* beside_in,
+    float* __restrict__ state, long slot_stride, const int32_t* __restrict__ seq_start, const int32_t* __restrict__ seq_slot,
+    float* __restrict__ read, float* beside, int H, int dim, int vdim, int tiles, float q_scale) {
+  constexpr int DIM = ML_SLICES * R;      // the rows of a column that the registers hold (dim <= DIM)
+  __shared__ float s_q[ML_STAGE][DIM];
+  __shared__ float s_k[ML_STAGE][DIM];    // times b_t already
+  __shared__ float s_v[ML_STAGE][ML_COLS];
+  __shared__ float s_a[ML_STAGE];
+  const int tile = blockIdx.x % tiles, unit = blockIdx.x / tiles;
+  const int head = unit % H, seq = unit / H;
+  const int row0 = seq_start[seq], rows = seq_start[seq + 1] - row0;
+  if (rows <= 0) return;
+  const int tid = threadIdx.x, c = tid / ML_SLICES, s = tid % ML_SLICES;
+  const int column = tile * ML_COLS + c;      // vdim is n's
+  const int head_floats = (vdim + 1) * dim + 1;
+  float* mine = state + (size_t)seq_slot[seq] * slot_stride + (size_t)head * head_floats + (size_t)column * dim;
+  float S[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int d = s + ML_SLICES * r;
+    S[r] = (column <= vdim && d < dim) ? mine[d] : 0.f;
+  }
+  // what this thread brings into a stage: row `c` of it, dimensions s + 16 r of q and k; the tile's value (c, s as row, column)
+  float next_q[R], next_k[R], next_v = 0.f, next_a = 1.f, next_b = 0.f;
+  auto ask = [&](int base) {
+    const int t = base + c;
+    const bool live = t < rows;
+    const T* x = proj + (size_t)(row0 + (live ? t : 0)) * row_stride + (size_t)head * dim;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const int d = s + ML_SLICES * r;
+      const bool there = live && d < dim;
+      next_q[r] = there ? to_f32(x[q_off + d]) : 0.f;
+      next_k[r] = there ? to_f32(x[k_off + d]) : 0.f;
+    }
+    const float* g = beside_in + ((size_t)(row0 + (live ? t : 0)) * H + head) * ML_BESIDE;
+    next_a = live ? g[0] : 1.f;
+    next_b = live ? g[1] : 0.f;
+    const int value = tile * ML_COLS + s;
+    next_v = 0.f;
+    if (live && value < vdim) next_v = to_f32(proj[(size_t)(row0 + t) * row_stride + v_off + (size_t)head * vdim + value]);
+    else if (live && value == vdim) next_v = 1.f;
+  };
+  ask(0);
+  for (int base = 0; base < rows; base += ML_STAGE) {
+    __syncthreads();      // the stage before has been walked by all
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      s_q[c][s + ML_SLICES * r] = next_q[r] * q_scale;
+      s_k[c][s + ML_SLICES * r] = next_k[r] * next_b;
+    }
+    s_v[c][s] = next_v;
+    if (s == 0) s_a[c] = next_a;
+    __syncthreads();
+    if (base + ML_STAGE < rows) ask(base + ML_STAGE);
+    const int live = rows - base < ML_STAGE ? rows - base : ML_STAGE;
+    for (int t = 0; t < live; ++t) {
+      const float a = s_a[t], v = s_v[t][c];
+      float acc = 0.f;
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const int d = s + ML_SLICES * r;
+        S[r] = fmaf(a, S[r], s_k[t][d] * v);
+        acc = fmaf(S[r], s_q[t][d], acc);
+      }
+      acc += __shfl_xor(acc, 8, BH_WAVE);
+      acc += __shfl_xor(acc, 4, BH_WAVE);
+      acc += __shfl_xor(acc, 2, BH_WAVE);
+      acc += __shfl_xor(acc, 1, BH_WAVE);
+      if (s == 0) {
+        const size_t row = (size_t)(row0 + base + t);
+        if (column < vdim) read[row * H * vdim + (size_t)head * vdim + column] = acc;
+        else if (column == vdim) beside[(row * H + head) * ML_BESIDE + 3] = acc;
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int d = s + ML_SLICES * r;
+    if (column <= vdim && d < dim) mine[d] = S[r];
+  }
+}
+
+// proj [n_rows][row_stride] holds a row's q and k (H heads of dim) and v (H heads of vdim) from q_off, k_off, v_off; beside
+// f32 [n_rows][H][4] as mlstm_gates left it (its fourth number, n . q, is written here); read f32 [n_rows][H * vdim].
+extern "C" int bh_mlstm_scan(const void* proj, int dtype, int row_stride, int q_off, int k_off, int v_off, float* beside, float* state,
+                             long slot_stride, const int32_t* seq_start, const int32_t* seq_slot, float* read, int n_seqs, int H, int dim,
+                             int vdim, hipStream_t stream) {
+  BH_REQUIRE(n_seqs > 0 && H > 0 && dim > 0 && vdim > 0, "mlstm_scan: sizes must be positive");
+  BH_REQUIRE(dim <= ML_SLICES * 32, "mlstm_scan: heads of %d key dimensions are above the limit of %d", dim, ML_SLICES * 32);
+  BH_REQUIRE((long)H * ((long)(vdim + 1) * dim + 1) <= slot_stride, "mlstm_scan: %d heads of %d x %d do not fit a slot's %ld floats", H, dim,
+             vdim, slot_stride);
+  BH_REQUIRE(q_off >= 0 && k_off >= 0 && v_off >= 0 && q_off + H * dim <= row_stride && k_off + H * dim <= row_stride &&
+                 v_off + H * vdim <= row_stride, "mlstm_scan: q, k and v lie outside a row of %d", row_stride);
+  const int tiles = (vdim + 1 + ML_COLS - 1) / ML_COLS;
+  BH_REQUIRE((long)n_seqs * H * tiles < (1L << 31), "mlstm_scan: too many workgroups");
+  const float q_scale = 1.0f / sqrtf((float)dim);
+  const int per = (dim + ML_SLICES - 1) / ML_SLICES;
+#define BH_ML(T, R)                                                                                                              \
+  mlstm_scan_kernel<T, R><<<n_seqs * H * tiles, ML_COLS * ML_SLICES, 0, stream>>>((const T*)proj, row_stride, q_off, k_off, v_off, beside, \
+                                                                               state, slot_stride, seq_start, seq_slot, read, beside, H, \
+                                                                               dim, vdim, tiles, q_scale)
+#define BH_ML_SIZES(T)              \
+  do {                              \
+    if (per <= 1) BH_ML(T, 1);      \
+    else if (per <= 2) BH_ML(T, 2); \
+    else if (per <= 4) BH_ML(T, 4); \
+    else if (per <= 8) BH_ML(T, 8); \
+    else if (per <= 16) BH_ML(T, 16); \
+    else BH_ML(T, 32);              \
+  } while (0)
+  if (dtype == BH_F32) BH_ML_SIZES(float);
+  else if (dtype == BH_BF16) BH_ML_SIZES(bf16_t);
+  else return bh_fail("mlstm_scan: unknown dtype %d", dtype);
+#undef BH_ML_SIZES
+#undef BH_ML
+  return bh_check_launch("mlstm_scan");
+}
+
+// ---- the read-out: division, norm of each head, weight, gate ----------------------------------------------------------
+// A wave a (row, head).
+template <typename T>
+__global__ __launch_bounds__(256) void mlstm_finish_kernel(const float* __restrict__ read, const float* __restrict__ beside,
+                                                           const T* __restrict__ gate, int gate_stride, int gate_first,
+                                                           const float* __restrict__ w, float eps, T* __restrict__ out, int n_rows, int H,
+                                                           int vdim, int out_block_rows) {
+  const int unit = blockIdx.x * (blockDim.x / BH_WAVE) + threadIdx.x / BH_WAVE, lane = threadIdx.x % BH_WAVE;
+  if (unit >= n_rows * H) return;
+  const int row = unit / H, head = unit % H;
+  const float* b = beside + (size_t)unit * ML_BESIDE;
+  const float inv = 1.0f / (fmaxf(fabsf(b[3]), expf(-b[2])) + 1e-6f);
+  const float* o = read + (size_t)row * H * vdim + (size_t)head * vdim;
+  float ss = 0.f;
+  for (int e = lane; e < vdim; e += BH_WAVE) {
+    const float v = o[e] * inv;
+    ss += v * v;
+  }
+  const float norm = 1.0f / sqrtf(wave_sum(ss) / (float)vdim + eps);
+  for (int e = lane; e < vdim; e += BH_WAVE) {
+    const int column = head * vdim + e;
+    const float g = to_f32(gate[(size_t)row * gate_stride + gate_first + column]);
+    const float y = o[e] * inv * norm * (w ? w[column] : 1.f) / (1.0f + expf(-g));
+    out[bh_rows_index(out_block_rows, row, column, H * vdim)] = from_f32<T>(y);
+  }
+}
+
+extern "C" int bh_mlstm_finish(const float* read, const float* beside, const void* gate, int dtype, int gate_stride, int gate_first,
+                               const float* w, float eps, void* out, int n_rows, int H, int vdim, int out_block_rows, hipStream_t stream) {
+  BH_REQUIRE(n_rows > 0 && H > 0 && vdim > 0, "mlstm_finish: sizes must be positive");
+  BH_REQUIRE(gate_first >= 0 && gate_first + H * vdim <= gate_stride, "mlstm_finish: the gate lies outside its row");
+  BH_REQUIRE(out_block_rows == 0 || ((out_block_rows == 8 || out_block_rows == 16) && (H * vdim) % 32 == 0 && dtype == BH_BF16),
+             "mlstm_finish: rows in blocks of %d of width %d are not written", out_block_rows, H * vdim);
+  const long units = (long)n_rows * H;
+  BH_REQUIRE((units + 3) / 4 < (1L << 31), "mlstm_finish: too many rows");
+  const int blocks = (int)((units + 3) / 4);
+  if (dtype == BH_F32)
+    mlstm_finish_kernel<float><<<blocks, 256, 0, stream>>>(read, beside, (const float*)gate, gate_stride, gate_first, w, eps, (float*)out,
+                                                         n_rows, H, vdim, out_block_rows);
+  else if (dtype == BH_BF16)
+    mlstm_finish_kernel<bf16_t><<<blocks, 256, 0, stream>>>(read, beside, (const bf16_t*)gate, gate_stride, gate_first, w, eps,
+                                                          (bf16_t*)out, n_rows, H, vdim, out_block_rows);
+  else
+    return bh_fail("mlstm_finish: unknown dtype %d", dtype);
+  return bh_check_launch("mlstm_finish");
+}

@@ -147,12 +147,12 @@ int bhp_qk_norm_rope_cache(const void* qkv, int dtype, void* q_out, const void* 
 int bhp_attention(const void* q, void* out, int dtype, const void* k_pages, const void* v_pages,
                   const int32_t* page_table, int table_stride, const int32_t* row_seq, const int32_t* positions,
                   int n_rows, int H, int KVH, int hd, float scale, int window, int kv_order, int pages) {
-  if (!known(dtype) || n_rows <= 0 || H <= 0 || KVH <= 0 || H % KVH || hd <= 0 || window < 0) return 1;
+  if (!known(dtype) || n_rows <= 0 || H <= 0 || KVH <= 0 || H % KVH || hd <= 0) return 1;
   const int G = H / KVH;
   std::vector<float> score;
   std::vector<double> value(hd);
   for (int r = 0; r < n_rows; ++r) {
-    const int pos = positions[r], first = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+    const int pos = positions[r], first = bh_first_visible(pos, window);
     if (pos < 0 || pos / BH_PAGE >= table_stride) return 2;
     score.assign(pos + 1 - first, 0.f);
     for (int h = 0; h < H; ++h) {

@@ -1,5 +1,7 @@
 // Small row-wise operations on the float32 residual and on logits:
 //   layernorm        (x - mean) / sqrt(var + eps) * w + b per row, optional row gather, rows or blocks of rows out
+//   sum_layernorm    h <- layernorm(alpha h + y) per row in place, and the same rounded for the product that reads it next
+//   gelu_tanh        out = gelu(x), tanh form, elementwise into rows or blocks of rows
 //   cast_concat      [a | b] per row from float32 into the activation type (b optional): the input of a product
 //   softcap          x <- cap * tanh(x / cap) in place
 //   rms_scale_add    h <- h + y / sqrt(mean(y^2) + eps) * w per row
@@ -43,6 +45,52 @@ extern "C" int bh_layernorm(const float* x, const int32_t* rows, const float* w,
   else
     return bh_fail("layernorm: unknown dtype %d", out_dtype);
   return bh_check_launch("layernorm");
+}
+
+// h <- ((s - mean) / sqrt(var + eps)) * w + b with s = alpha * h + y: the norm stands behind the sum.  One workgroup a
+// row; a thread meets the same elements in all three passes, so the sum can stand in h's own place between them.  With
+// `rounded` the result also goes out in the activation type (rows or blocks of rows), for the product that reads it next.
+template <typename TO>
+__global__ __launch_bounds__(256) void sum_layernorm_kernel(float* __restrict__ h, const float* __restrict__ y, float alpha,
+                                                            const float* __restrict__ w, const float* __restrict__ b,
+                                                            TO* __restrict__ rounded, int width, float eps, int out_block_rows) {
+  __shared__ float scratch[8];
+  const int r = blockIdx.x;
+  float* row = h + (size_t)r * width;
+  const float* add = y + (size_t)r * width;
+  float sum = 0.f;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    const float s = fmaf(alpha, row[i], add[i]);
+    row[i] = s;
+    sum += s;
+  }
+  const float mean = block_sum(sum, scratch) / (float)width;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    const float d = row[i] - mean;
+    ss += d * d;
+  }
+  const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / (float)width + eps);
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    const float v = (row[i] - mean) * inv * w[i] + (b ? b[i] : 0.f);
+    row[i] = v;
+    if (rounded) rounded[bh_rows_index(out_block_rows, r, i, width)] = from_f32<TO>(v);
+  }
+}
+
+extern "C" int bh_sum_layernorm(float* h, const float* y, float alpha, const float* w, const float* b, void* rounded,
+                                int out_dtype, int n_rows, int width, float eps, int out_block_rows, hipStream_t stream) {
+  BH_REQUIRE(n_rows > 0 && width > 0, "sum_layernorm: sizes must be positive");
+  BH_REQUIRE(h != y, "sum_layernorm: the sublayer's result stands apart from the residual");
+  BH_REQUIRE(out_block_rows == 0 || (rounded && (out_block_rows == 8 || out_block_rows == 16) && width % 32 == 0 && out_dtype == BH_BF16),
+             "sum_layernorm: rows in blocks of %d of width %d are not written", out_block_rows, width);
+  if (rounded == nullptr || out_dtype == BH_F32)
+    sum_layernorm_kernel<float><<<n_rows, 256, 0, stream>>>(h, y, alpha, w, b, (float*)rounded, width, eps, out_block_rows);
+  else if (out_dtype == BH_BF16)
+    sum_layernorm_kernel<bf16_t><<<n_rows, 256, 0, stream>>>(h, y, alpha, w, b, (bf16_t*)rounded, width, eps, out_block_rows);
+  else
+    return bh_fail("sum_layernorm: unknown dtype %d", out_dtype);
+  return bh_check_launch("sum_layernorm");
 }
 
 template <typename TO>
@@ -106,6 +154,30 @@ extern "C" int bh_rms_scale_add(float* h, const float* y, const float* w, int n_
 
 __device__ inline float gelu_tanh(float z) {
   return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void gelu_tanh_kernel(const T* __restrict__ x, T* __restrict__ out, int width, size_t total, int block_rows) {
+  const size_t at = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (at >= total) return;
+  const size_t to = block_rows ? (size_t)bh_rows_index(block_rows, (int)(at / width), (int)(at % width), width) : at;
+  out[to] = from_f32<T>(gelu_tanh(to_f32(x[at])));
+}
+
+extern "C" int bh_gelu_tanh(const void* x, void* out, int dtype, int n_rows, int width, int out_block_rows, hipStream_t stream) {
+  BH_REQUIRE(n_rows > 0 && width > 0, "gelu_tanh: nothing to do");
+  BH_REQUIRE(out_block_rows == 0 || ((out_block_rows == 8 || out_block_rows == 16) && dtype == BH_BF16 && width % 32 == 0 && x != out),
+             "gelu_tanh: rows in blocks of %d need bfloat16, a width that is a multiple of 32 (got %d) and an output of their own",
+             out_block_rows, width);
+  const size_t total = (size_t)n_rows * width;
+  const size_t blocks = (total + 255) / 256;
+  BH_REQUIRE(blocks <= 2147483647u, "gelu_tanh: too many elements");
+  if (dtype == BH_F32)
+    gelu_tanh_kernel<float><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>((const float*)x, (float*)out, width, total, out_block_rows);
+  else if (dtype == BH_BF16)
+    gelu_tanh_kernel<bf16_t><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>((const bf16_t*)x, (bf16_t*)out, width, total, out_block_rows);
+  else return bh_fail("gelu_tanh: unknown dtype %d", dtype);
+  return bh_check_launch("gelu_tanh");
 }
 
 // A row's token is tokens[row], or fed[token_src[row]] where token_src is given and not negative (a token chosen on the

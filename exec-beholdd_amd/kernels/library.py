@@ -175,6 +175,12 @@ class KernelSizes:
             "bh_rotate_heads": [p, ctypes.c_long, i, i, p, ctypes.c_long, i, i, i, p, i, p, i, i, i, p],
             "bh_layernorm": [p, p, p, p, p, i, i, i, f, i, p],
             "bh_cast_concat": [p, p, p, i, i, i, i, p],
+            "bh_sum_layernorm": [p, p, f, p, p, p, i, i, i, f, i, p],
+            "bh_gelu_tanh": [p, p, i, i, i, i, p],
+            "bh_head_norm_rope_write": [p, i, i, i, p, p, p, f, p, i, p, p, p, p, p, p, i, i, i, i, i, i, i, i, i, p],
+            "bh_mlstm_gates": [p, p, f, p, ctypes.c_long, i, p, p, p, i, i, p],
+            "bh_mlstm_scan": [p, i, i, i, i, i, p, p, ctypes.c_long, p, p, p, i, i, i, i, p],
+            "bh_mlstm_finish": [p, p, p, i, i, i, p, f, p, i, i, i, i, p],
             "bh_softcap": [p, ctypes.c_long, f, p],
             "bh_rms_scale_add": [p, p, p, i, i, f, p],
             "bh_gelu_gate_table": [p, i, p, p, p, p, i, i, i, p, i, i, i, p],
@@ -685,13 +691,18 @@ class HipKernels(KernelSizes):
             raise KernelError(f"{what}: the page table must be [sequences, pages]")
 
     def attention(self, q, out, k_pages, v_pages, page_table, row_seq, positions, n_heads, n_kv_heads, head_dim,
-                  scale, window=0, layout=None):
+                  scale, window=0, layout=None, chunk=0):
         """out[row, head] = softmax(q . K * scale) V over the keys of the row's sequence that the row
-        may see: positions max(0, p - window + 1) .. p (window 0 = all).  `layout`, when given,
+        may see: positions max(0, p - window + 1) .. p with a window, p - p % chunk .. p with chunks (counted from
+        the sequence's position 0), else 0 .. p; not both.  `layout`, when given,
         says how rows group into sequences (seq_start int32 [n_seqs + 1] on the device, n_seqs,
         max_rows_per_seq, max_position), which the matrix-core kernel needs; rows of one sequence
         are consecutive and in position order."""
         n_rows = q.shape[0]
+        if window < 0 or chunk < 0 or (window and chunk):
+            raise KernelError(f"attention: a window ({window}) or chunks ({chunk}) of a positive count of positions, not both")
+        if chunk:
+            window = -int(chunk)      # the kernels' one number for both (csrc/layout.h: bh_first_visible)
         if q.shape != (n_rows, n_heads * head_dim) or tuple(out.shape) != tuple(q.shape) or out.dtype != q.dtype:
             raise KernelError(f"attention: shapes q {tuple(q.shape)}, out {tuple(out.shape)} do not fit")
         # the matrix-core kernels write blocks themselves: of 16 rows in steps of many columns, of 8 or 16 otherwise
@@ -701,7 +712,7 @@ class HipKernels(KernelSizes):
                     int(layout.n_seqs), int(layout.max_rows_per_seq), n_heads, n_kv_heads, int(layout.max_position)))):
             rows_out = torch.empty(tuple(q.shape), dtype=q.dtype, device=self.device)   # this step's kernel writes rows
             self.attention(q, rows_out, k_pages, v_pages, page_table, row_seq, positions, n_heads, n_kv_heads, head_dim,
-                           scale, window, layout)
+                           scale, max(window, 0), layout, chunk)
             self.to_blocked(rows_out, out)
             return
         if n_heads % n_kv_heads != 0:
@@ -964,6 +975,114 @@ class HipKernels(KernelSizes):
             self._ptr(x, "layernorm x", (torch.float32,)), self._ptr(rows, "layernorm rows", (torch.int32,), True),
             self._ptr(weight, "layernorm weight", (torch.float32,)), self._ptr(bias, "layernorm bias", (torch.float32,), True),
             self._ptr(out, "layernorm out"), _code(out, "layernorm out"), n_rows, width, float(eps), _block_rows(out), self._stream()))
+
+    def sum_layernorm(self, hidden, y, alpha, weight, bias, eps, rounded=None):
+        """hidden[r] <- layernorm(alpha * hidden[r] + y[r]) * weight + bias in place (all f32, the variance as the mean of
+        the squared deviations); `rounded` [n, D], if given, takes the same in its own type, in rows or blocks of rows."""
+        n_rows, width = hidden.shape
+        if tuple(y.shape) != (n_rows, width) or weight.shape != (width,) or (bias is not None and bias.shape != (width,)) \
+                or (rounded is not None and tuple(rounded.shape) != (n_rows, width)):
+            raise KernelError(f"sum_layernorm: shapes hidden {tuple(hidden.shape)}, y {tuple(y.shape)} do not fit")
+        self._check(self.lib.bh_sum_layernorm(
+            self._ptr(hidden, "sum_layernorm hidden", (torch.float32,)), self._ptr(y, "sum_layernorm y", (torch.float32,)), float(alpha),
+            self._ptr(weight, "sum_layernorm weight", (torch.float32,)), self._ptr(bias, "sum_layernorm bias", (torch.float32,), True),
+            self._ptr(rounded, "sum_layernorm rounded", None, True), _code(rounded, "sum_layernorm rounded") if rounded is not None else F32,
+            n_rows, width, float(eps), _block_rows(rounded) if rounded is not None else 0, self._stream()))
+
+    def gelu_tanh(self, x, out=None):
+        """out <- x/2 (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))); in place without `out`, which may be `BlockedRows`."""
+        out = x if out is None else out
+        if x.dim() != 2 or tuple(out.shape) != tuple(x.shape) or out.dtype != x.dtype:
+            raise KernelError(f"gelu_tanh: shapes {tuple(x.shape)} -> {tuple(out.shape)} do not fit")
+        self._check(self.lib.bh_gelu_tanh(self._ptr(x, "gelu_tanh x"), self._ptr(out, "gelu_tanh out"), _code(x, "gelu_tanh x"),
+                                          x.shape[0], x.shape[1], _block_rows(out), self._stream()))
+
+    def head_norm_rope_write(self, proj, first, bias, q_weight, k_weight, eps, freq, turned, positions, row_seq, q_out, k_pages,
+                             v_pages, page_table, n_heads, n_kv_heads, dim, vdim, pad, write_kv):
+        """From column `first` of every row of `proj` [n, P]: q (H heads of dim), k (G of dim), v (G of vdim), plus `bias` (f32
+        over those channels, or None); every head of q and k normed by its own root mean square times q_weight / k_weight
+        (f32 [dim], both or None); dimensions i and i + turned/2 of every head of q and k turned by position * freq[i];
+        q -> q_out [n, H pad], k and v into the cache pages as heads of `pad` (see csrc/head_norm_attention.hip)."""
+        n_rows = proj.shape[0]
+        channels = (n_heads + n_kv_heads) * dim + n_kv_heads * vdim
+        if tuple(q_out.shape) != (n_rows, n_heads * pad) or q_out.dtype != proj.dtype or first < 0 or first + channels > proj.shape[1]:
+            raise KernelError(f"head_norm_rope_write: shapes proj {tuple(proj.shape)}, q_out {tuple(q_out.shape)} do not fit")
+        if (q_weight is None) != (k_weight is None) or (q_weight is not None and (q_weight.shape != (dim,) or k_weight.shape != (dim,))):
+            raise KernelError("head_norm_rope_write: one norm weight per dimension of a head, for queries and keys alike")
+        if bias is not None and bias.shape != (channels,):
+            raise KernelError(f"head_norm_rope_write: a bias per channel ({channels}), got {tuple(bias.shape)}")
+        if positions.shape != (n_rows,) or row_seq.shape != (n_rows,):
+            raise KernelError("head_norm_rope_write: positions and row_seq must have one entry per row")
+        if turned and (freq is None or freq.shape != (turned // 2,)):
+            raise KernelError("head_norm_rope_write: one frequency per turned pair")
+        self._check_pages(k_pages, v_pages, page_table, n_kv_heads, pad, q_out.dtype, "head_norm_rope_write")
+        f32, i32 = (torch.float32,), (torch.int32,)
+        self._check(self.lib.bh_head_norm_rope_write(
+            self._ptr(proj, "proj"), _code(proj, "proj"), proj.shape[1], int(first), self._ptr(bias, "bias", f32, True),
+            self._ptr(q_weight, "q norm", f32, True), self._ptr(k_weight, "k norm", f32, True), float(eps),
+            self._ptr(freq, "frequencies", f32, True), int(turned), self._ptr(positions, "positions", i32),
+            self._ptr(row_seq, "row_seq", i32), self._ptr(q_out, "q_out"), self._ptr(k_pages, "k_pages"), self._ptr(v_pages, "v_pages"),
+            self._ptr(page_table, "page_table", i32), page_table.shape[1], n_rows, n_heads, n_kv_heads, dim, vdim, pad,
+            self.kv_order(k_pages.dtype, pad), int(bool(write_kv)), self._stream()))
+
+    # ---- a matrix memory with exponential gates, as a recurrence over a float32 state ----
+    MLSTM_BESIDE = 4      # floats a row and head beside the read-out: a_t, b_t, m_t, n_t . q_t
+
+    @staticmethod
+    def mlstm_state_floats(n_heads, dim, vdim) -> int:
+        """Floats of a sequence's state: per head vdim + 1 columns of dim (the last one n), then m."""
+        return n_heads * ((vdim + 1) * dim + 1)
+
+    def mlstm_gates(self, pre, bias, cap, state, seq_start, seq_slot, beside, n_heads, dim, vdim):
+        """beside[row, head] = (a_t, b_t, m_t, .) from the gates' pre-activations pre f32 [n, 2 H] (input gates, then forget
+        gates) plus bias f32 [2 H]: i = cap tanh(x_i / cap), f = logsigmoid(cap tanh(x_f / cap)), m_t = max(f + m_(t-1), i),
+        a = exp(f + m_(t-1) - m_t), b = exp(i - m_t); the rows of sequence b (seq_start) in order from the m of state row
+        seq_slot[b], which is moved on.  state f32 [slots, mlstm_state_floats]."""
+        n_rows = pre.shape[0]
+        n_seqs = seq_slot.shape[0]
+        if tuple(pre.shape) != (n_rows, 2 * n_heads) or tuple(beside.shape) != (n_rows, n_heads * self.MLSTM_BESIDE) \
+                or state.dim() != 2 or state.shape[1] < self.mlstm_state_floats(n_heads, dim, vdim) \
+                or tuple(seq_start.shape) != (n_seqs + 1,) or (bias is not None and tuple(bias.shape) != (2 * n_heads,)):
+            raise KernelError(f"mlstm_gates: shapes pre {tuple(pre.shape)}, state {tuple(state.shape)}, beside {tuple(beside.shape)} "
+                              f"do not fit {n_heads} heads of {dim} x {vdim} and {n_seqs} sequences")
+        f32, i32 = (torch.float32,), (torch.int32,)
+        self._check(self.lib.bh_mlstm_gates(
+            self._ptr(pre, "mlstm gates", f32), self._ptr(bias, "mlstm gate bias", f32, True), float(cap),
+            self._ptr(state, "mlstm state", f32), state.shape[1], (vdim + 1) * dim + 1, self._ptr(seq_start, "seq_start", i32),
+            self._ptr(seq_slot, "seq_slot", i32), self._ptr(beside, "mlstm beside", f32), n_seqs, n_heads, self._stream()))
+
+    def mlstm_scan(self, proj, q_off, k_off, v_off, beside, state, seq_start, seq_slot, read, n_heads, dim, vdim):
+        """For every sequence of the step and head: S <- a_t S + b_t k_t [v_t | 1]^T over the sequence's rows in order (a_t, b_t
+        from `beside`), read[row, head] = S^T q_t / sqrt(dim) over the vdim value columns and beside[row, head, 3] = the same
+        over the column of ones (n . q); q, k, v are the row's slices of `proj` [n, P] from q_off, k_off, v_off."""
+        n_rows = proj.shape[0]
+        n_seqs = seq_slot.shape[0]
+        if tuple(read.shape) != (n_rows, n_heads * vdim) or tuple(beside.shape) != (n_rows, n_heads * self.MLSTM_BESIDE) \
+                or state.dim() != 2 or state.shape[1] < self.mlstm_state_floats(n_heads, dim, vdim) \
+                or tuple(seq_start.shape) != (n_seqs + 1,):
+            raise KernelError(f"mlstm_scan: shapes proj {tuple(proj.shape)}, state {tuple(state.shape)}, read {tuple(read.shape)} "
+                              f"do not fit {n_heads} heads of {dim} x {vdim} and {n_seqs} sequences")
+        f32, i32 = (torch.float32,), (torch.int32,)
+        self._check(self.lib.bh_mlstm_scan(
+            self._ptr(proj, "mlstm proj"), _code(proj, "mlstm proj"), proj.shape[1], int(q_off), int(k_off), int(v_off),
+            self._ptr(beside, "mlstm beside", f32), self._ptr(state, "mlstm state", f32), state.shape[1],
+            self._ptr(seq_start, "seq_start", i32), self._ptr(seq_slot, "seq_slot", i32), self._ptr(read, "mlstm read", f32),
+            n_seqs, n_heads, dim, vdim, self._stream()))
+
+    def mlstm_finish(self, read, beside, proj, gate_off, weight, eps, out, n_heads, vdim):
+        """out[r, h] = rms-normed over vdim (read[r, h] / (max(|n . q|, exp(-m)) + 1e-6)) * weight * sigmoid(proj[r, gate_off ..]);
+        out [n, H vdim] in the type of `proj`, rows or `BlockedRows`."""
+        n_rows = read.shape[0]
+        width = n_heads * vdim
+        if tuple(read.shape) != (n_rows, width) or tuple(beside.shape) != (n_rows, n_heads * self.MLSTM_BESIDE) \
+                or tuple(out.shape) != (n_rows, width) or proj.shape[0] != n_rows or out.dtype != proj.dtype \
+                or (weight is not None and tuple(weight.shape) != (width,)):
+            raise KernelError(f"mlstm_finish: shapes read {tuple(read.shape)}, proj {tuple(proj.shape)}, out {tuple(out.shape)} do not fit")
+        f32 = (torch.float32,)
+        self._check(self.lib.bh_mlstm_finish(
+            self._ptr(read, "mlstm read", f32), self._ptr(beside, "mlstm beside", f32), self._ptr(proj, "mlstm gate"),
+            _code(proj, "mlstm gate"), proj.shape[1], int(gate_off), self._ptr(weight, "mlstm norm weight", f32, True), float(eps),
+            self._ptr(out, "mlstm out"), n_rows, n_heads, vdim, _block_rows(out), self._stream()))
 
     def cast_concat(self, a, b, out):
         """out[r] = [a[r] | b[r]] in out's type; a, b f32 [n, D] (b may be None), out [n, 2 D] (or [n, D])."""

@@ -3,7 +3,9 @@
 The configuration supplies, layer by layer, the names of the parts (`layer_kinds()`) and the
 order of execution (`schedule()`): a list of (layer index, cache entry index).  A layer may be
 named twice (its weights run twice, each run with a cache entry of its own), and an entry may
-be shared: the first run that names an entry writes it, later runs read it.
+be shared: the first run that names an entry writes it, later runs read it.  A layer that the
+configuration gives no parts (`layer_kinds()` has None in its place: it runs another layer's) keeps
+its number, so that the other layers' tensor names stay the file's, and no run may name it.
 The whole-model order follows the reference: embed, every layer, then final norm and head on
 the rows that are asked for (crates/beholdd-model/src/qwen3moe/forward.rs:811-915, :1416-1455).
 """
@@ -29,6 +31,8 @@ class DecoderModel:
         for layer, entry in self.schedule:
             if not 0 <= layer < len(self.blocks):
                 raise ValueError(f"the schedule names layer {layer}, the model has {len(self.blocks)}")
+            if self.blocks[layer] is None:
+                raise ValueError(f"the schedule names layer {layer}, which has no parts of its own")
             if entry < 0:
                 raise ValueError("cache entry indices are not negative")
         # entry -> need, and which scheduled run owns (writes) each entry
@@ -57,20 +61,24 @@ class DecoderModel:
 
     def parts(self):
         opening = [part for part in (self.residual, self.pass_input) if part is not None]
-        return [self.embedding, *opening, *self.shared_parts, *self.blocks, self.final_norm, self.head]
+        return [self.embedding, *opening, *self.shared_parts, *self.own_blocks(), self.final_norm, self.head]
+
+    def own_blocks(self) -> list:
+        """The blocks that exist: every layer but those that run another layer's parts."""
+        return [block for block in self.blocks if block is not None]
 
     @property
     def graph_safe(self):
         """True when a decode step of this model may be captured as a HIP graph: every part's
         forward depends on the step's device tensors only."""
         return all(getattr(part, "graph_safe", False)
-                   for part in (self.embedding, *self.blocks, self.final_norm, self.head)
+                   for part in (self.embedding, *self.own_blocks(), self.final_norm, self.head)
                    ) and all(getattr(part, "graph_safe", False) for part in (self.residual, self.pass_input) if part is not None)
 
     @property
     def graph_safe_rows(self) -> int:
         """Up to how many tokens per sequence a captured step may bring (every sequence the same number)."""
-        return graph_rows_allowed((self.embedding, *self.blocks, self.final_norm, self.head))
+        return graph_rows_allowed((self.embedding, *self.own_blocks(), self.final_norm, self.head))
 
     def tensor_specs(self):
         return [spec for part in self.parts() for spec in part.tensor_specs()]
@@ -96,7 +104,7 @@ class DecoderModel:
         for part in (self.residual, self.pass_input):
             if hasattr(part, "working_bytes"):
                 total += part.working_bytes(step)
-        widest = max([block.working_bytes(step) for block in self.blocks if hasattr(block, "working_bytes")], default=0)
+        widest = max([block.working_bytes(step) for block in self.own_blocks() if hasattr(block, "working_bytes")], default=0)
         last = 0
         if hasattr(self.final_norm, "working_bytes"):
             last += self.final_norm.working_bytes(step, rows=step.wanted)
@@ -107,7 +115,7 @@ class DecoderModel:
     def unaccounted_parts(self) -> list:
         """Names of parts that do not say what their forward allocates (the byte plan lists them)."""
         names = [type(part).__name__ for part in (self.embedding, self.final_norm, self.head) if not hasattr(part, "working_bytes")]
-        for block in self.blocks:
+        for block in self.own_blocks():
             names += block.unaccounted_parts() if hasattr(block, "unaccounted_parts") else [type(block).__name__]
         return sorted(set(names))
 
@@ -163,7 +171,7 @@ def build_decoder(config, position_encoding="rope", layer_prefix: str = "model.l
     embedding = make_embedding(config) if make_embedding else Embedding(config.vocab, config.hidden, embedding_name)
     blocks = []
     for index, kinds in enumerate(config.layer_kinds()):
-        blocks.append(BLOCKS.get(kinds.block)(config, index, layer_prefix.format(index), kinds, shared))
+        blocks.append(BLOCKS.get(kinds.block)(config, index, layer_prefix.format(index), kinds, shared) if kinds is not None else None)
     final_norm = NORMS.get(final_norm_kind)(config, config.hidden, final_norm_name, shared)
     if make_head:
         head = make_head(config, embedding)

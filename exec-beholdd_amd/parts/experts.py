@@ -1,7 +1,8 @@
 """Routed experts: a mixture of small gated feed-forward layers of which every token uses a few, and a shared one.
 
-    z = Wr h + br                       router logits, float32 (h in the activation type)
-    chosen = the `top` largest of z;  their weights = softmax over the chosen logits alone
+    z = Wr h + br                       router logits, float32 (h in the activation type); the bias is optional
+    chosen = the `top` largest of z;  their weights = softmax over the chosen logits alone (which is also what the
+                                        chosen ones' shares of a softmax over all experts are once divided by their sum)
     expert(h) = Wd (g' * sigmoid(alpha g') * (u' + 1)),  g' = min(Wg h, limit),  u' = clamp(Wu h, -limit, limit)
     out = sum over chosen of weight * expert(h)  +  shared(h)        (the shared expert has the same form and runs for all)
 
@@ -77,18 +78,21 @@ class RoutedExperts:
                               # operands through the L2), the products per expert cost about 25 us each and then run faster
 
     def __init__(self, hidden: int, n_experts: int, top: int, ff: int, limit: float, prefix: str, shared: ClampedGLU | None = None,
-                 alpha: float = GATE_SLOPE):
+                 alpha: float = GATE_SLOPE, router_bias: bool = True):
         if not 1 <= top <= n_experts:
             raise ValueError(f"a row uses 1 to {n_experts} experts, got {top}")
         self.hidden, self.n_experts, self.top, self.ff = int(hidden), int(n_experts), int(top), int(ff)
         self.limit, self.alpha, self.prefix, self.shared = float(limit), float(alpha), prefix, shared
         self.router = Linear(hidden, n_experts, prefix + "router")
+        self.has_router_bias = bool(router_bias)
         self.router_bias = self.w_gate_up = self.w_down = None
         self.for_products = None      # per expert (gate and up, down) as the matrix products take them
         self.in_one_launch = False    # a prompt's products run as one launch over all experts (kernels.experts_products)
 
     def tensor_specs(self):
-        specs = self.router.tensor_specs() + [TensorSpec(self.prefix + "router.b", (self.n_experts,), "linear")]
+        specs = self.router.tensor_specs()
+        if self.has_router_bias:
+            specs.append(TensorSpec(self.prefix + "router.b", (self.n_experts,), "linear"))
         for e in range(self.n_experts):
             specs += [TensorSpec(f"{self.prefix}e{e}.gate", (self.ff, self.hidden), "linear"),
                       TensorSpec(f"{self.prefix}e{e}.up", (self.ff, self.hidden), "linear"),
@@ -97,7 +101,7 @@ class RoutedExperts:
 
     def load(self, get):
         self.router.load(get)
-        self.router_bias = get(self.prefix + "router.b").to(torch.float32).contiguous()
+        self.router_bias = get(self.prefix + "router.b").to(torch.float32).contiguous() if self.has_router_bias else None
         first = get(f"{self.prefix}e0.gate")
         self.w_gate_up = torch.empty((self.n_experts, 2 * self.ff, self.hidden), dtype=first.dtype, device=first.device)
         self.w_down = torch.empty((self.n_experts, self.hidden, self.ff), dtype=first.dtype, device=first.device)
@@ -199,4 +203,5 @@ class RoutedExperts:
 def _build_routed_experts(config, layer_index, prefix, shared):
     sizes = config.layers[layer_index].mlp
     common = ClampedGLU(config.hidden, sizes.shared.ff, sizes.shared.limit, prefix + "mlp.shared.") if sizes.shared is not None else None
-    return RoutedExperts(config.hidden, sizes.experts, sizes.top, sizes.expert.ff, sizes.expert.limit, prefix + "mlp.", shared=common)
+    return RoutedExperts(config.hidden, sizes.experts, sizes.top, sizes.expert.ff, sizes.expert.limit, prefix + "mlp.", shared=common,
+                         router_bias=getattr(sizes, "router_bias", True))

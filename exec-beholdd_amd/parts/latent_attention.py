@@ -11,7 +11,10 @@ latent into the head's values, by one small matrix per head each (`heads_linear`
 paged attention kernels' own case of one key/value head of size kv_rank + rot_dim shared by all query heads, with
 key [c | k_r] and value [c | 0]; prompts and decode steps take the same path, so a position's result does not
 depend on the cut.  The rotation turns the first `rotation.dims` dimensions of the rot_dim part, dimension i with
-i + dims/2, by position * base^(-2i/dims) (angles in float32, no table, no longest position).
+i + dims/2, by position * base^(-2i/dims) (angles in float32, no table, no longest position).  A model without a
+rotated part has rot_dim 0 and no rotation; with a `window` a query sees the last `window` positions only (its own
+among them) and the cache gives older pages back; with `gate` the heads' values are multiplied by sigmoid(Wg x) ahead
+of the output projection, the gate being one more slice of the stacked projection.
 Every size and constant is a constructor parameter.
 """
 
@@ -31,16 +34,21 @@ class LatentAttention:
     writes_fresh = True    # forward(..., fresh=True) writes its result instead of adding it
 
     def __init__(self, hidden: int, n_heads: int, dim: int, rot_dim: int, vdim: int, kv_rank: int, scale: float,
-                 rotation: RotaryFrequencies, norm_eps: float, prefix: str):
-        if rotation.dims > rot_dim:
+                 rotation: RotaryFrequencies | None, norm_eps: float, prefix: str, window: int = 0, gate: bool = False):
+        if (rotation.dims if rotation is not None else 0) > rot_dim:
             raise ValueError(f"the rotation turns {rotation.dims} dimensions, the rotated part has {rot_dim}")
+        if window < 0:
+            raise ValueError(f"a window is a count of positions (0: all), got {window}")
         self.hidden, self.n_heads, self.dim, self.rot_dim = int(hidden), int(n_heads), int(dim), int(rot_dim)
         self.vdim, self.kv_rank, self.scale = int(vdim), int(kv_rank), float(scale)
         self.rotation, self.norm_eps, self.prefix = rotation, float(norm_eps), prefix
+        self.window, self.gate = int(window), bool(gate)
         self.q_head = self.dim + self.rot_dim                 # a head of the projected query
         self.kv_head = self.kv_rank + self.rot_dim            # the one cached key/value head
         self.down_off = self.n_heads * self.q_head            # where [c_raw | k_r] begins in a projected row
-        self.proj = Linear(hidden, [self.n_heads * self.q_head, self.kv_head], [prefix + "q", prefix + "dkv"])
+        self.gate_off = self.down_off + self.kv_head         # where the gate begins, if there is one
+        gate_width, gate_name = ([self.n_heads * self.vdim], [prefix + "g"]) if self.gate else ([], [])
+        self.proj = Linear(hidden, [self.n_heads * self.q_head, self.kv_head] + gate_width, [prefix + "q", prefix + "dkv"] + gate_name)
         self.out = Linear(self.n_heads * self.vdim, hidden, prefix + "o")
         self.latent_weight = self.key_up = self.value_up = self.frequencies = None
 
@@ -62,18 +70,18 @@ class LatentAttention:
         # kv_rank -> vdim through Wuv transposed
         self.key_up = get(self.prefix + "uk").view(self.n_heads, self.dim, self.kv_rank).contiguous()
         self.value_up = get(self.prefix + "uv").view(self.n_heads, self.vdim, self.kv_rank).transpose(1, 2).contiguous()
-        self.frequencies = self.rotation.frequencies(self.latent_weight.device)
+        self.frequencies = self.rotation.frequencies(self.latent_weight.device) if self.rotation is not None else None
 
     def prepare(self, kernels):
         self.proj.prepare(kernels)
         self.out.prepare(kernels)
 
     def cache_need(self):
-        return CacheNeed(kind="kv", kv_heads=1, head_dim=self.kv_head)
+        return CacheNeed(kind="kv", kv_heads=1, head_dim=self.kv_head, window=self.window)
 
     def working_bytes(self, step) -> int:
         total = self.proj.working_bytes(step, step.rows) + 2 * step.matrix(step.rows, self.n_heads * self.kv_head)
-        total += step.matrix(step.rows, self.n_heads * self.vdim)
+        total += (2 if self.gate else 1) * step.matrix(step.rows, self.n_heads * self.vdim)
         if step.sizes is not None:
             total += step.sizes.attention_working_bytes(step.rows, step.seqs, step.max_rows_per_seq, self.n_heads, 1,
                                                         self.kv_head, step.max_position, step.act_size)
@@ -81,20 +89,31 @@ class LatentAttention:
 
     def forward(self, ctx, x, hidden, cache, then_norm=None, fresh=False):
         k = ctx.kernels
-        heads, rank, turned = self.n_heads, self.kv_rank, self.rotation.dims
+        heads, rank, turned = self.n_heads, self.kv_rank, self.rotation.dims if self.rotation is not None else 0
         proj = self.proj.forward(ctx, x)
         query = ctx.new_activations(ctx.n_rows, heads * self.kv_head)
         # one launch: c and k_r into the cache, and the heads' rotated query parts into their places
-        k.latent_write(proj, self.down_off, self.latent_weight, self.norm_eps, self.frequencies, turned, ctx.positions,
-                       ctx.row_seq, cache.k_pages, cache.v_pages, cache.page_table, rank, self.rot_dim, write=cache.writes,
-                       query=query, query_head=self.kv_head, query_first=rank, source_head=self.q_head, source_first=self.dim,
-                       n_heads=heads)
+        if self.rot_dim:
+            k.latent_write(proj, self.down_off, self.latent_weight, self.norm_eps, self.frequencies, turned, ctx.positions,
+                           ctx.row_seq, cache.k_pages, cache.v_pages, cache.page_table, rank, self.rot_dim, write=cache.writes,
+                           query=query, query_head=self.kv_head, query_first=rank, source_head=self.q_head, source_first=self.dim,
+                           n_heads=heads)
+        elif cache.writes:
+            k.latent_write(proj, self.down_off, self.latent_weight, self.norm_eps, None, 0, ctx.positions, ctx.row_seq,
+                           cache.k_pages, cache.v_pages, cache.page_table, rank, 0)
         k.heads_linear(proj, self.q_head, 0, self.key_up, query, self.kv_head, 0, heads)
         attended = ctx.new_activations(ctx.n_rows, heads * self.kv_head)
         k.attention(query, attended, cache.k_pages, cache.v_pages, cache.page_table, ctx.row_seq, ctx.positions,
-                    heads, 1, self.kv_head, self.scale, 0, layout=ctx)
-        values = ctx.new_activations(ctx.n_rows, heads * self.vdim, reader=self.out.reader())
-        k.heads_linear(attended, self.kv_head, 0, self.value_up, values, self.vdim, 0, heads)
+                    heads, 1, self.kv_head, self.scale, self.window, layout=ctx)
+        if self.gate:
+            values = ctx.new_activations(ctx.n_rows, heads * self.vdim)
+            k.heads_linear(attended, self.kv_head, 0, self.value_up, values, self.vdim, 0, heads)
+            gated = ctx.new_activations(ctx.n_rows, heads * self.vdim, reader=self.out.reader())
+            k.gate_heads(values, self.vdim, proj, self.gate_off, gated, heads, self.vdim)
+            values = gated
+        else:
+            values = ctx.new_activations(ctx.n_rows, heads * self.vdim, reader=self.out.reader())
+            k.heads_linear(attended, self.kv_head, 0, self.value_up, values, self.vdim, 0, heads)
         self.out.forward(ctx, values, out=hidden, accumulate=not fresh)
         return None
 
@@ -102,5 +121,7 @@ class LatentAttention:
 @MIXERS.register("latent_attention")
 def _build_latent_attention(config, layer_index, prefix, shared):
     sizes = config.layers[layer_index].mixer
+    rotation = RotaryFrequencies(sizes.rot_dims, sizes.rot_base) if sizes.rot_dims else None
     return LatentAttention(config.hidden, sizes.heads, sizes.dim, sizes.rot_dim, sizes.vdim, sizes.kv_rank, sizes.scale,
-                           RotaryFrequencies(sizes.rot_dims, sizes.rot_base), config.rms_eps, prefix + "mix.")
+                           rotation, config.rms_eps, prefix + "mix.", window=getattr(sizes, "window", 0),
+                           gate=getattr(sizes, "gate", False))

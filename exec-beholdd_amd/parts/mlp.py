@@ -91,6 +91,22 @@ class SquaredReLU:
         self.down.forward(ctx, activated, out=hidden, accumulate=not fresh)
 
 
+class GeluTanh(SquaredReLU):
+    """The same with the tanh form of GELU between the two matrices: out = Wd gelu(Wu x),
+    gelu(z) = z/2 (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))."""
+
+    def forward(self, ctx, x, hidden, fresh=False):
+        inner = self.up.forward(ctx, x)
+        activated = ctx.new_activations(inner.shape[0], self.inner, reader=self.down.reader())
+        ctx.kernels.gelu_tanh(inner, activated)
+        self.down.forward(ctx, activated, out=hidden, accumulate=not fresh)
+
+
+@FEED_FORWARDS.register("gelu_tanh")
+def _build_gelu_tanh(config, layer_index, prefix, shared):
+    return GeluTanh(config.hidden, config.layers[layer_index].mlp.ff, prefix + "mlp.")
+
+
 @FEED_FORWARDS.register("squared_relu")
 def _build_squared_relu(config, layer_index, prefix, shared):
     return SquaredReLU(config.hidden, config.layers[layer_index].ff, prefix + "mlp.")

@@ -114,6 +114,18 @@ class LayerNorm:
     def working_bytes(self, step, rows: int | None = None, reader=None) -> int:
         return step.matrix(step.rows if rows is None else rows, self.width, reader=reader)
 
+    def sum_forward(self, ctx, hidden, result, alpha: float, reader=None, rounded: bool = True):
+        """hidden <- norm(alpha * hidden + result), row by row and in place: the weighted sum, the statistics and the result
+        are float32.  Returns what a sublayer that reads the new residual takes as its input: the residual itself where
+        the activations are float32, else a copy rounded to the activation type, written by the same kernel (in the form
+        `reader` reads fastest); None when `rounded` says that nobody reads one."""
+        if ctx.act_dtype == torch.float32:
+            ctx.kernels.sum_layernorm(hidden, result, alpha, self.weight, self.bias, self.eps, None)
+            return hidden if rounded else None
+        out = ctx.new_activations(hidden.shape[0], self.width, reader=reader) if rounded else None
+        ctx.kernels.sum_layernorm(hidden, result, alpha, self.weight, self.bias, self.eps, out)
+        return out
+
 
 @NORMS.register("layernorm")
 def _build_layernorm(config, width, name, shared):
