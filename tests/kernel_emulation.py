@@ -75,15 +75,16 @@ class TorchKernels:
             v_pages[page, :, :, pos % PAGE] = v[row].to(v_pages.dtype)
 
     def attention(self, q, out, k_pages, v_pages, page_table, row_seq, positions, n_heads, n_kv_heads, head_dim,
-                  scale, window=0, layout=None):
+                  scale, window=0, layout=None, chunk=0):
         self.calls.append("attention")
+        assert not (window and chunk)
         n_rows = q.shape[0]
         group = n_heads // n_kv_heads
         qh = q.float().reshape(n_rows, n_heads, head_dim)
         result = torch.empty_like(qh)
         for row in range(n_rows):
             pos, seq = int(positions[row]), int(row_seq[row])
-            first = max(0, pos - window + 1) if window else 0
+            first = max(0, pos - window + 1) if window else (pos - pos % chunk if chunk else 0)
             index = torch.arange(first, pos + 1)
             pages = page_table[seq, index // PAGE].long()
             keys = k_pages[pages, :, index % PAGE, :].float()      # [n, kv_heads, head_dim]
@@ -305,6 +306,108 @@ class TorchKernels:
         n = attended.shape[0]
         a = attended.float().reshape(n, n_heads, pad)[..., :vdim].reshape(n, n_heads * vdim)
         out.copy_((a * torch.sigmoid(gate[:, gate_first:gate_first + n_heads * vdim].float())).to(out.dtype))
+
+    # ---- norm behind the sum, GELU, heads normed one by one, a matrix memory ----
+    def sum_layernorm(self, hidden, y, alpha, weight, bias, eps, rounded=None):
+        self.calls.append("sum_layernorm")
+        total = alpha * hidden.double() + y.double()
+        centred = total - total.mean(-1, keepdim=True)
+        result = centred / torch.sqrt((centred ** 2).mean(-1, keepdim=True) + eps) * weight.double()
+        if bias is not None:
+            result = result + bias.double()
+        hidden.copy_(result.float())
+        if rounded is not None:
+            rounded.copy_(result.to(rounded.dtype))
+
+    def gelu_tanh(self, x, out=None):
+        self.calls.append("gelu_tanh")
+        z = x.double()
+        (x if out is None else out).copy_((0.5 * z * (1.0 + torch.tanh(0.7978845608028654 * (z + 0.044715 * z ** 3)))).to(x.dtype))
+
+    def head_norm_rope_write(self, proj, first, bias, q_weight, k_weight, eps, freq, turned, positions, row_seq, q_out, k_pages,
+                             v_pages, page_table, n_heads, n_kv_heads, dim, vdim, pad, write_kv):
+        self.calls.append("head_norm_rope_write")
+        n = proj.shape[0]
+        q_width, k_width, v_width = n_heads * dim, n_kv_heads * dim, n_kv_heads * vdim
+        x = proj[:, first:first + q_width + k_width + v_width].float()
+        if bias is not None:
+            x = x + bias.float()
+        q = x[:, :q_width].reshape(n, n_heads, dim)
+        k = x[:, q_width:q_width + k_width].reshape(n, n_kv_heads, dim)
+        v = x[:, q_width + k_width:].reshape(n, n_kv_heads, vdim)
+        if q_weight is not None:
+            rms = lambda t, w: (t.double() / torch.sqrt((t.double() ** 2).mean(-1, keepdim=True) + eps) * w.double()).float()
+            q, k = rms(q, q_weight), rms(k, k_weight)
+        q, k = self._turn(q, freq, turned, positions), self._turn(k, freq, turned, positions)
+        wide = torch.zeros(n, n_heads, pad)
+        wide[..., :dim] = q
+        q_out.copy_(wide.reshape(n, n_heads * pad).to(q_out.dtype))
+        if not write_kv:
+            return
+        for row in range(n):
+            pos, seq = int(positions[row]), int(row_seq[row])
+            page = int(page_table[seq, pos // PAGE])
+            k_pages[page, :, pos % PAGE, :] = 0
+            v_pages[page, :, :, pos % PAGE] = 0
+            k_pages[page, :, pos % PAGE, :dim] = k[row].to(k_pages.dtype)
+            v_pages[page, :, :vdim, pos % PAGE] = v[row].to(v_pages.dtype)
+
+    MLSTM_BESIDE = 4
+
+    @staticmethod
+    def mlstm_state_floats(n_heads, dim, vdim):
+        return n_heads * ((vdim + 1) * dim + 1)
+
+    def mlstm_gates(self, pre, bias, cap, state, seq_start, seq_slot, beside, n_heads, dim, vdim):
+        self.calls.append("mlstm_gates")
+        x = pre.float() + (bias.float() if bias is not None else 0.0)
+        gate_i = cap * torch.tanh(x[:, :n_heads] / cap)
+        gate_f = torch.nn.functional.logsigmoid(cap * torch.tanh(x[:, n_heads:] / cap))
+        head_floats = (vdim + 1) * dim + 1
+        out = beside.view(-1, n_heads, 4)
+        for b in range(seq_slot.shape[0]):
+            slot = int(seq_slot[b])
+            m = state[slot].view(n_heads, head_floats)[:, -1].clone()
+            for row in range(int(seq_start[b]), int(seq_start[b + 1])):
+                new = torch.maximum(gate_f[row] + m, gate_i[row])
+                out[row, :, 0] = torch.exp(gate_f[row] + m - new)
+                out[row, :, 1] = torch.exp(gate_i[row] - new)
+                out[row, :, 2] = new
+                m = new
+            state[slot].view(n_heads, head_floats)[:, -1] = m
+
+    def mlstm_scan(self, proj, q_off, k_off, v_off, beside, state, seq_start, seq_slot, read, n_heads, dim, vdim):
+        self.calls.append("mlstm_scan")
+        n = proj.shape[0]
+        q = proj[:, q_off:q_off + n_heads * dim].float().reshape(n, n_heads, dim) * (1.0 / (dim ** 0.5))
+        k = proj[:, k_off:k_off + n_heads * dim].float().reshape(n, n_heads, dim)
+        v = torch.cat([proj[:, v_off:v_off + n_heads * vdim].float().reshape(n, n_heads, vdim), torch.ones(n, n_heads, 1)], dim=-1)
+        head_floats = (vdim + 1) * dim + 1
+        factors = beside.view(n, n_heads, 4)
+        for b in range(seq_slot.shape[0]):
+            slot = int(seq_slot[b])
+            held = state[slot].view(n_heads, head_floats)[:, :-1].reshape(n_heads, vdim + 1, dim)      # column-major: [column][dim]
+            S = held.clone().double()
+            for row in range(int(seq_start[b]), int(seq_start[b + 1])):
+                a, w = factors[row, :, 0].double(), factors[row, :, 1].double()
+                S = a[:, None, None] * S + w[:, None, None] * v[row].double()[:, :, None] * k[row].double()[:, None, :]
+                got = torch.einsum("hcd,hd->hc", S, q[row].double()).float()
+                read[row] = got[:, :vdim].reshape(-1)
+                factors[row, :, 3] = got[:, vdim]
+                S = S.float().double()
+            state[slot].view(n_heads, head_floats)[:, :-1] = S.float().reshape(n_heads, -1)
+
+    def mlstm_finish(self, read, beside, proj, gate_off, weight, eps, out, n_heads, vdim):
+        self.calls.append("mlstm_finish")
+        n = read.shape[0]
+        factors = beside.view(n, n_heads, 4)
+        under = torch.maximum(factors[:, :, 3].abs(), torch.exp(-factors[:, :, 2])) + 1e-6
+        o = read.view(n, n_heads, vdim).double() / under.double()[:, :, None]
+        o = (o / torch.sqrt((o ** 2).mean(-1, keepdim=True) + eps)).reshape(n, n_heads * vdim)
+        if weight is not None:
+            o = o * weight.double()
+        gate = torch.sigmoid(proj[:, gate_off:gate_off + n_heads * vdim].double())
+        out.copy_((o * gate).to(out.dtype))
 
     # ---- a state-space recurrence ----
     def ssm_scan(self, xbc, proj, dt_first, dt_bias, a_log, d_skip, state, state_offset, seq_start, seq_slot, out, n_heads, vdim,
