@@ -63,6 +63,12 @@ def parse():
                              "experts, a per-layer token input, a looped stretch) at layer sizes of real models beside Qwen3 at "
                              "equal width and as many layer runs: prefill and decode tokens per second of both, and every kernel "
                              "of the new design beside its like with the fraction of its roofline; prints one JSON line and exits")
+    parser.add_argument("--dupidra", action="store_true",
+                        help="the Dupidra design (gated attention within chunks, windowed attention over a cached latent, a matrix "
+                             "memory with exponential gates, routed experts and dense GELU feed-forwards behind post-norm sums, "
+                             "layers that run another layer's tensors) at layer sizes of real models beside Pudorax and Qwen3 at "
+                             "equal width and as many layer runs: prefill and decode tokens per second, and every kernel of the "
+                             "new design beside its like with the fraction of its roofline; prints one JSON line and exits")
     parser.add_argument("--sampling", action="store_true",
                         help="time the selection kernel on 1, 8 and 64 rows of 151,936 logits (greedy, at a temperature, with "
                              "top-k, with top-p on rows of three spreads, with both), print the microseconds and exit")
@@ -622,6 +628,187 @@ def pudorax_bench(args, torch):
     return 0
 
 
+# ---- the Dupidra design beside Pudorax and Qwen3 at equal width and as many layer runs ---------------------------
+
+def dupidra_config(width, heads, vocab, experts=32, top=4, chunk=8192, window=4096, rank=256):
+    """Eight layer runs of which two run an earlier layer's tensors: attention with heads of 128, four query heads to a
+    key/value head, a rotation over half a head and chunks of `chunk` positions; attention over a latent of `rank` within a
+    window; matrix memories with keys of 64 and values of 128 a head; `experts` experts of 3/8 of the width of which `top`
+    are used in all layers but one, whose feed-forward is dense and three times the width."""
+    mlp = {"kind": "moe", "router": {"experts": experts, "top": top}, "expert": {"ff": 3 * width // 8, "limit": 7.0}}
+    attention = {"type": "attention", "mlp": mlp,
+                 "mixer": {"heads": heads, "kv_heads": max(heads // 4, 1), "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                           "mask": {"size": chunk}, "rot": {"base": 1000000.0, "dims": 64}}}
+    latent = {"type": "latent_attention", "mlp": mlp,
+              "mixer": {"heads": heads, "dim": 128, "vdim": 128, "kv_rank": rank, "scale": 128 ** -0.5, "mask": {"size": window}}}
+    memory = {"type": "mlstm", "mlp": mlp, "mixer": {"heads": heads, "dim": 64, "vdim": 128, "gate_cap": 15.0}}
+    first_memory = dict(memory, mlp={"kind": "dense", "ff": 3 * width})
+    return {"architecture": "Dupidra", "vocab": vocab, "width": width, "postln_alpha": 2.0, "norm": {"eps": 1e-6},
+            "layers": [attention, first_memory, latent, dict(attention, weights_of=0), memory, latent, dict(memory, weights_of=4),
+                       attention]}
+
+
+def dupidra_kernels(K, torch, width, heads, context, rank=256):
+    """Every kernel that the design brought and its like among the other models', alone, at a prompt of 2,048 rows and at a
+    decode step of 8 rows over `context` cached tokens: microseconds and the fraction of the roofline (the slower of its bytes
+    at the HBM peak and its operations at the peak of the units it runs on)."""
+    from types import SimpleNamespace
+    bf16, dev = torch.bfloat16, "cuda:0"
+    dim = vdim = 128
+    page = K.page_size
+    out = {}
+
+    def note(name, us, n_bytes, flops=0.0, peak=PEAK_FLOPS["fp32"]):
+        floor = max(n_bytes / (PEAK_HBM_GBS * 1e9), flops / peak) * 1e6
+        out[name] = {"us": round(us, 1), "roofline_us": round(floor, 2), "fraction": round(floor / us, 3)}
+
+    def pages_for(n_seqs, length, kv_heads, head):
+        per = -(-length // page)
+        k_pages = torch.randn(n_seqs * per, kv_heads, page, head, device=dev).to(bf16)
+        v_pages = torch.randn(n_seqs * per, kv_heads, head, page, device=dev).to(bf16)
+        table = torch.arange(n_seqs * per, dtype=torch.int32, device=dev).view(n_seqs, per).contiguous()
+        return k_pages, v_pages, table
+
+    kv_heads = max(heads // 4, 1)
+    ones = torch.ones(width, device=dev)
+    for rows, seqs, past, tag in ((2048, 1, 0, "prompt of 2,048"), (8, 8, context - 1, f"decode of 8 at {context}")):
+        each = rows // seqs
+        starts = torch.arange(0, rows + 1, each, dtype=torch.int32, device=dev)
+        slots = torch.arange(seqs, dtype=torch.int32, device=dev)
+        positions = (torch.arange(rows, dtype=torch.int32, device=dev) % each + past).contiguous()
+        row_seq = (torch.arange(rows, dtype=torch.int32, device=dev) // each).contiguous()
+        layout = SimpleNamespace(seq_start=starts, n_seqs=seqs, max_rows_per_seq=each, max_position=past + each - 1)
+        keys_seen = seqs * (past + each) if each == 1 else each * (each + 1) // 2
+        # -- the norm behind the sum, beside the norms that stand ahead
+        hidden, result = torch.randn(rows, width, device=dev), torch.randn(rows, width, device=dev)
+        normed = torch.empty(rows, width, device=dev, dtype=bf16)
+        us = timed(lambda: K.sum_layernorm(hidden, result, 2.0, ones, ones, 1e-6, normed), torch)
+        note(f"sum_layernorm, {tag}", us, 3 * hidden.numel() * 4 + normed.numel() * 2)
+        us = timed(lambda: K.layernorm(hidden, ones, ones, 1e-6, normed), torch)
+        note(f"pudorax layernorm, {tag}", us, hidden.numel() * 4 + normed.numel() * 2)
+        us = timed(lambda: K.rmsnorm(hidden, ones, 1e-6, normed), torch)
+        note(f"qwen3 rmsnorm, {tag}", us, hidden.numel() * 4 + normed.numel() * 2)
+        # -- attention: biases, head norms, rotation and cache write; the attention within chunks; the gate
+        q_w, k_w = heads * dim, kv_heads * dim
+        proj = torch.randn(rows, 2 * q_w + 2 * k_w, device=dev).to(bf16)
+        bias = torch.randn(q_w + 2 * k_w, device=dev)
+        head_weight, freq = torch.ones(dim, device=dev), torch.ones(32, device=dev)
+        k_pages, v_pages, table = pages_for(seqs, past + each, kv_heads, dim)
+        q_out = torch.empty(rows, heads * dim, device=dev, dtype=bf16)
+        us = timed(lambda: K.head_norm_rope_write(proj, 0, bias, head_weight, head_weight, 1e-6, freq, 64, positions, row_seq, q_out, k_pages,
+                                                  v_pages, table, heads, kv_heads, dim, vdim, dim, True), torch)
+        note(f"head_norm_rope_write, {tag}", us, 2 * rows * (q_w + 2 * k_w) * 2)
+        qkv = torch.randn(rows, q_w + 2 * k_w, device=dev).to(bf16)
+        cos = torch.ones(past + each, dim // 2, device=dev)
+        us = timed(lambda: K.qk_norm_rope_cache(qkv, q_out, head_weight, head_weight, 1e-6, cos, cos, positions, row_seq, k_pages, v_pages,
+                                                table, heads, kv_heads, dim, True, past + each - 1), torch)
+        note(f"qwen3 qk_norm_rope_cache, {tag}", us, 2 * qkv.numel() * 2)
+        attended = torch.empty_like(q_out)
+        chunk = -(-(past + each) // page) * page      # the whole context is one chunk: as many keys as Qwen3's attention reads
+        us = timed(lambda: K.attention(q_out, attended, k_pages, v_pages, table, row_seq, positions, heads, kv_heads, dim, dim ** -0.5, 0,
+                                       layout=layout, chunk=chunk), torch)
+        attention_bytes = 2 * seqs * (past + each) * kv_heads * dim * 2 + 2 * q_out.numel() * 2
+        note(f"attention within a chunk ({heads} heads on {kv_heads} of {dim}), {tag}", us, attention_bytes, 4.0 * keys_seen * heads * dim,
+             PEAK_FLOPS["bf16"])
+        us = timed(lambda: K.attention(q_out, attended, k_pages, v_pages, table, row_seq, positions, heads, kv_heads, dim, dim ** -0.5, 0,
+                                       layout=layout), torch)
+        note(f"qwen3 attention ({heads} heads on {kv_heads} of {dim}), {tag}", us, attention_bytes, 4.0 * keys_seen * heads * dim,
+             PEAK_FLOPS["bf16"])
+        gated = torch.empty(rows, heads * vdim, device=dev, dtype=bf16)
+        us = timed(lambda: K.gate_heads(attended, dim, proj, q_w + 2 * k_w, gated, heads, vdim), torch)
+        note(f"gate_heads, {tag}", us, 3 * gated.numel() * 2)
+        # -- attention over the latent, without a rotated part, within a window
+        qd = torch.randn(rows, heads * dim + rank + heads * vdim, device=dev).to(bf16)
+        lk, lv, ltable = pages_for(seqs, past + each, 1, rank)
+        latent_weight = torch.ones(rank, device=dev)
+        us = timed(lambda: K.latent_write(qd, heads * dim, latent_weight, 1e-6, None, 0, positions, row_seq, lk, lv, ltable, rank, 0), torch)
+        note(f"latent_write without a rotated part, {tag}", us, rows * rank * 2 * 3)
+        key_up = torch.randn(heads, dim, rank, device=dev).to(bf16)
+        query = torch.empty(rows, heads * rank, device=dev, dtype=bf16)
+        us = timed(lambda: K.heads_linear(qd, dim, 0, key_up, query, rank, 0, heads), torch)
+        note(f"heads_linear (queries into the latent), {tag}", us, key_up.numel() * 2 + rows * heads * (dim + rank) * 2,
+             2.0 * rows * heads * dim * rank, PEAK_FLOPS["bf16"])
+        seen_window = min(4096, past + each)
+        lat_out = torch.empty_like(query)
+        us = timed(lambda: K.attention(query, lat_out, lk, lv, ltable, row_seq, positions, heads, 1, rank, dim ** -0.5, 4096, layout=layout), torch)
+        note(f"attention over the latent within a window of 4,096 ({heads} heads on one of {rank}), {tag}", us,
+             2 * seqs * seen_window * rank * 2 + 2 * query.numel() * 2, 4.0 * (seqs * seen_window if each == 1 else keys_seen) * heads * rank,
+             PEAK_FLOPS["bf16"])
+        value_up = torch.randn(heads, rank, vdim, device=dev).to(bf16)
+        values = torch.empty(rows, heads * vdim, device=dev, dtype=bf16)
+        us = timed(lambda: K.heads_linear(lat_out, rank, 0, value_up, values, vdim, 0, heads), torch)
+        note(f"heads_linear (latents into values), {tag}", us, value_up.numel() * 2 + rows * heads * (rank + vdim) * 2,
+             2.0 * rows * heads * rank * vdim, PEAK_FLOPS["bf16"])
+        # -- the matrix memory beside the recurrences of the other designs
+        m_dim = 64
+        m_proj = torch.randn(rows, 2 * heads * m_dim + 2 * heads * vdim, device=dev).to(bf16)
+        pre = torch.randn(rows, 2 * heads, device=dev)
+        gate_bias = torch.ones(2 * heads, device=dev)
+        m_state = torch.zeros(seqs, K.mlstm_state_floats(heads, m_dim, vdim), device=dev)
+        beside = torch.empty(rows, 4 * heads, device=dev)
+        read = torch.empty(rows, heads * vdim, device=dev)
+        us = timed(lambda: K.mlstm_gates(pre, gate_bias, 15.0, m_state, starts, slots, beside, heads, m_dim, vdim), torch)
+        note(f"mlstm_gates, {tag}", us, pre.numel() * 4 + beside.numel() * 4)
+        us = timed(lambda: K.mlstm_scan(m_proj, 0, heads * m_dim, 2 * heads * m_dim, beside, m_state, starts, slots, read, heads, m_dim, vdim), torch)
+        note(f"mlstm_scan, {tag}", us, 2 * m_state.numel() * 4 + rows * heads * (2 * m_dim + vdim) * 2 + read.numel() * 4,
+             3.0 * rows * heads * m_dim * (vdim + 1))
+        m_out = torch.empty(rows, heads * vdim, device=dev, dtype=bf16)
+        m_weight = torch.ones(heads * vdim, device=dev)
+        us = timed(lambda: K.mlstm_finish(read, beside, m_proj, 2 * heads * m_dim + heads * vdim, m_weight, 1e-6, m_out, heads, vdim), torch)
+        note(f"mlstm_finish, {tag}", us, read.numel() * 4 + 2 * m_out.numel() * 2)
+        l_proj = torch.randn(rows, 4 * heads * dim, device=dev).to(bf16)
+        l_state = torch.zeros(seqs, heads, dim, vdim, device=dev)
+        decay = torch.full((heads,), 0.99, device=dev)
+        mixed = torch.empty(rows, heads * vdim, device=dev)
+        us = timed(lambda: K.lightning_scan(l_proj, 0, heads * dim, 2 * heads * dim, l_state, decay, starts, slots, mixed, heads, dim, vdim), torch)
+        note(f"gokazen lightning_scan, {tag}", us, 2 * l_state.numel() * 4 + rows * 3 * heads * dim * 2 + mixed.numel() * 4,
+             4.0 * rows * heads * dim * vdim)
+        l_gated = torch.empty(rows, heads * vdim, device=dev, dtype=bf16)
+        us = timed(lambda: K.gated_rmsnorm(mixed, l_proj, 3 * heads * dim, m_weight, 1e-6, l_gated), torch)
+        note(f"gokazen gated_rmsnorm, {tag}", us, mixed.numel() * 4 + 2 * l_gated.numel() * 2)
+        # -- the dense feed-forward's activation beside the others'
+        inner = torch.randn(rows, 3 * width, device=dev).to(bf16)
+        activated = torch.empty_like(inner)
+        us = timed(lambda: K.gelu_tanh(inner, activated), torch)
+        note(f"gelu_tanh, {tag}", us, 2 * inner.numel() * 2)
+        us = timed(lambda: K.relu_squared(inner, activated), torch)
+        note(f"gokazen relu_squared, {tag}", us, 2 * inner.numel() * 2)
+    return out
+
+
+def dupidra_bench(args, torch):
+    from beholdd.engine import Engine, random_model_on_device
+
+    device, points = "cuda:0", []
+    t = min(args.prefill_tokens, args.context)
+    for width, heads in ((2048, 16), (4096, 32)):
+        trio = {"dupidra": dupidra_config(width, heads, 32768),
+                "pudorax": pudorax_config(width, heads, 32768),
+                "qwen3": dict(QWEN3_8B, num_hidden_layers=8, hidden_size=width, num_attention_heads=heads,
+                              num_key_value_heads=heads // 4, intermediate_size=3 * width, vocab_size=32768)}
+        point = {"width": width, "heads": heads, "layer_runs": 8}
+        for name, config in trio.items():
+            model = random_model_on_device(config, seed=0, dtype="bfloat16", device=device)
+            engine = Engine(model=model, dtype="bfloat16", max_tokens=args.batch * (-(-args.context // 64) * 64),
+                            max_slots=args.batch, device=device)
+            parameters = sum(int(np_prod(spec.shape)) for spec in model.tensor_specs())
+            seconds, _ = decode_run(engine, args.batch, args.context, args.steps, args.warmup, torch)
+            prefill = prefill_run(engine, t, torch)
+            point[name] = {"parameters": parameters, "decode_ms_per_step": round(seconds * 1e3, 4),
+                           "decode_tok_per_s": round(args.batch / seconds, 1), "prefill_ms": round(prefill * 1e3, 3),
+                           "prefill_tok_per_s": round(t / prefill, 1)}
+            kernels = engine.kernels
+            del engine, model
+            torch.cuda.empty_cache()
+        points.append(point)
+    line = {"metric": f"Dupidra beside Pudorax and Qwen3 at equal width and as many layer runs: decode tok/s @ batch {args.batch}, context {args.context}; prefill of {t} tokens",
+            "unit": "tok/s", "value": points[-1]["dupidra"]["decode_tok_per_s"], "dtype": "bf16", "data": "synthetic", "n_gpus": 1,
+            "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "points": points,
+            "kernels": dupidra_kernels(kernels, torch, 4096, 32, args.context)}
+    print(json.dumps(line))
+    return 0
+
+
 def np_prod(shape):
     total = 1
     for axis in shape:
@@ -645,6 +832,8 @@ def main():
         return gokazen_bench(args, torch)
     if args.pudorax:
         return pudorax_bench(args, torch)
+    if args.dupidra:
+        return dupidra_bench(args, torch)
 
     from beholdd.engine import Engine, random_model_on_device
 

@@ -38,7 +38,9 @@ __global__ __launch_bounds__(BH_WAVE) void mlstm_gates_kernel(const float* __res
     float before = 0.f, mine = 0.f;
     const int steps = rows - base < BH_WAVE ? rows - base : BH_WAVE;
     for (int s = 0; s < steps; ++s) {
-      const float f_s = __shfl(gate_f, s, BH_WAVE), i_s = __shfl(gate_i, s, BH_WAVE);
+      // (s is the same in all lanes: a lane's value is read straight from its register)
+      const float f_s = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(gate_f), s));
+      const float i_s = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(gate_i), s));
       const float next = fmaxf(f_s + m, i_s);
       if (s == lane) {
         before = m;

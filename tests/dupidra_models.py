@@ -96,6 +96,11 @@ DEEP = _with_borrowers({
                mlstm(4, 32, 32, 12.0, mlp=moe(8, 4, 32, 1.0)),
                attention(8, 2, 32, 32, 0.18, chunk=33, rot_dims=8, base=1000.0, mlp=dense(200))],
 }, [(3, 1), (4, 0), (5, 2), (6, 1)])
+# The same layers with a residual that weighs little beside the sublayers (with matrices of twice the usual size): the
+# logits come from the embedding table too, so a model whose residual dominates predicts its last token over and over,
+# and greedy continuations would say nothing.
+GENERATING = dict(json.loads(json.dumps(MIXED)), postln_alpha=0.4)
+GENERATING_GAIN = 2.0
 CONFIGS = {"mixed": MIXED, "plain": PLAIN, "edges": EDGES, "deep": DEEP}
 
 

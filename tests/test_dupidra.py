@@ -275,11 +275,14 @@ def test_pages_behind_a_chunk_or_a_window_are_given_back(folders):
     engine.free_slot(slot)
 
 
-def test_greedy_generation_through_the_entry_point(folders):
-    folder, config, weights = folders("edges")
+def test_greedy_generation_through_the_entry_point(tmp_path):
+    config = dm.GENERATING
+    weights = dm.random_weights(config, 5, gain=dm.GENERATING_GAIN)
+    folder = dm.write_model(tmp_path / "generating", config, weights)
     prompts = schedules.random_requests(config["vocab"], [1, 9, 30], seed=6)
     engine = make_engine(folder)
     results = engine.generate(prompts, max_new_tokens=[6, 5, 6])
+    assert len({token for r in results for token in r.token_ids}) >= 6      # the continuations vary
     for prompt, result, n in zip(prompts, results, [6, 5, 6]):
         assert result.token_ids == plain.greedy(config, weights, prompt, n)
     engine.cache.check_invariants()
