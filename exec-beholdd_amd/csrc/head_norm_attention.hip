@@ -12,14 +12,16 @@
 
 #define HN_WAVES 4
 
-// A workgroup a row, a wave a head at a time: the heads of q, then those of k, then those of v.  The head stands in the
-// wave's own stretch of LDS between the statistic and the rotation, which needs a dimension's mate.
+// A workgroup a row and a stretch of `per_group` heads (the heads of q, then those of k, then those of v, numbered through), a
+// wave a head at a time.  The head stands in the wave's own stretch of LDS between the statistic and the rotation, which
+// needs a dimension's mate.  Few rows: a stretch is one head a wave, so that a decode step's heads run side by side.
 template <typename T>
 __global__ __launch_bounds__(HN_WAVES * BH_WAVE) void head_norm_rope_write_kernel(
     const T* __restrict__ proj, int row_stride, int first, const float* __restrict__ bias, const float* __restrict__ wq,
     const float* __restrict__ wk, float eps, const float* __restrict__ freq, int turned, const int32_t* __restrict__ positions,
     const int32_t* __restrict__ row_seq, T* __restrict__ q_out, T* __restrict__ k_pages, T* __restrict__ v_pages,
-    const int32_t* __restrict__ page_table, int table_stride, int H, int G, int dim, int vdim, int pad, int kv_order, int write) {
+    const int32_t* __restrict__ page_table, int table_stride, int H, int G, int dim, int vdim, int pad, int kv_order, int write,
+    int per_group) {
   extern __shared__ float lds[];      // the cosines and sines of the row's turned pairs, then a head of `dim` floats a wave
   const int row = blockIdx.x, wave = threadIdx.x / BH_WAVE, lane = threadIdx.x % BH_WAVE;
   const int half = turned / 2;
@@ -39,7 +41,8 @@ __global__ __launch_bounds__(HN_WAVES * BH_WAVE) void head_norm_rope_write_kerne
   const int token = pos % BH_PAGE;
   if (write) page = page_table[(size_t)row_seq[row] * table_stride + pos / BH_PAGE];
   const int heads = write ? H + 2 * G : H;
-  for (int unit = wave; unit < heads; unit += HN_WAVES) {
+  const int stretch_end = ((int)blockIdx.y + 1) * per_group < heads ? ((int)blockIdx.y + 1) * per_group : heads;
+  for (int unit = blockIdx.y * per_group + wave; unit < stretch_end; unit += HN_WAVES) {
     if (unit >= H + G) {      // a head of values: the bias, and zeros beyond vdim
       const int head = unit - H - G, at = q_width + k_width + head * vdim;
       T* values = v_pages + ((size_t)page * G + head) * BH_PAGE * pad;
@@ -100,11 +103,15 @@ extern "C" int bh_head_norm_rope_write(const void* proj, int dtype, int row_stri
              "head_norm_rope_write: cache order %d does not exist for head size %d", kv_order, pad);
   const size_t lds = (size_t)(turned + HN_WAVES * dim) * sizeof(float);
   BH_REQUIRE(lds <= 48 * 1024, "head_norm_rope_write: heads of %d dimensions do not fit the local memory", dim);
+  const int heads = write ? H + 2 * G : H;
+  const int per_group = n_rows >= 4 * bh_compute_units() ? 4 * HN_WAVES : HN_WAVES;      // many rows fill the chip by themselves
+  const dim3 grid(n_rows, (heads + per_group - 1) / per_group);
+  BH_REQUIRE(grid.y <= 65535, "head_norm_rope_write: too many heads");
 #define BH_HN(T)                                                                                                                  \
-  head_norm_rope_write_kernel<T><<<n_rows, HN_WAVES * BH_WAVE, lds, stream>>>((const T*)proj, row_stride, first, bias, wq, wk, eps, freq, \
-                                                                             turned, positions, row_seq, (T*)q_out, (T*)k_pages,  \
-                                                                             (T*)v_pages, page_table, table_stride, H, G, dim, vdim, \
-                                                                             pad, kv_order, write)
+  head_norm_rope_write_kernel<T><<<grid, HN_WAVES * BH_WAVE, lds, stream>>>((const T*)proj, row_stride, first, bias, wq, wk, eps, freq, \
+                                                                           turned, positions, row_seq, (T*)q_out, (T*)k_pages,    \
+                                                                           (T*)v_pages, page_table, table_stride, H, G, dim, vdim, \
+                                                                           pad, kv_order, write, per_group)
   if (dtype == BH_F32) BH_HN(float);
   else if (dtype == BH_BF16) BH_HN(bf16_t);
   else return bh_fail("head_norm_rope_write: unknown dtype %d", dtype);

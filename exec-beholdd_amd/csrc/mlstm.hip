@@ -15,8 +15,11 @@
 #define ML_BESIDE 4      // floats a row and head beside the read-out: a_t, b_t, m_t, n_t . q_t
 
 // ---- the gates -------------------------------------------------------------------------------------------------
-// A wave a (sequence, head).  64 rows at a time: every lane makes its row's two logarithms, then all lanes walk the 64
-// steps of m together (a step needs the one before), each keeping its own row's.
+// A wave a (sequence, head), 64 rows at a time, a lane a row.  A step of the maximum is the map x -> max(x + f, i); two steps
+// in a row are again such a map, (f1, i1) then (f2, i2) = (f1 + f2, max(i1 + f2, i2)), so the 64 maps are put together by a
+// prefix over the lanes in six exchanges and every lane applies its own to the m the block started from.  The sums of f
+// are added up in another order than one step after the other would; m only says by how much the state is scaled, and the
+// factors a and b are made from the same m's that are stored, so the state times exp(m) does not feel it.
 __global__ __launch_bounds__(BH_WAVE) void mlstm_gates_kernel(const float* __restrict__ pre, const float* __restrict__ bias, float cap,
                                                               float* __restrict__ state, long slot_stride, int head_floats,
                                                               const int32_t* __restrict__ seq_start, const int32_t* __restrict__ seq_slot,
@@ -28,32 +31,32 @@ __global__ __launch_bounds__(BH_WAVE) void mlstm_gates_kernel(const float* __res
   const float bias_i = bias ? bias[head] : 0.f, bias_f = bias ? bias[H + head] : 0.f, inv_cap = 1.0f / cap;
   for (int base = 0; base < rows; base += BH_WAVE) {
     const int t = base + lane;
-    float gate_i = 0.f, gate_f = 0.f;
+    float gate_i = -INFINITY, gate_f = 0.f;      // a row beyond the end is the map that changes nothing
     if (t < rows) {
       const float* x = pre + (size_t)(row0 + t) * 2 * H;
       gate_i = cap * tanhf((x[head] + bias_i) * inv_cap);
       const float z = cap * tanhf((x[H + head] + bias_f) * inv_cap);
       gate_f = fminf(z, 0.f) - log1pf(expf(-fabsf(z)));      // log(sigmoid(z)) without overflow
     }
-    float before = 0.f, mine = 0.f;
-    const int steps = rows - base < BH_WAVE ? rows - base : BH_WAVE;
-    for (int s = 0; s < steps; ++s) {
-      // (s is the same in all lanes: a lane's value is read straight from its register)
-      const float f_s = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(gate_f), s));
-      const float i_s = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(gate_i), s));
-      const float next = fmaxf(f_s + m, i_s);
-      if (s == lane) {
-        before = m;
-        mine = next;
+    float sum_f = gate_f, top_i = gate_i;      // the map of rows base .. t put together
+#pragma unroll
+    for (int off = 1; off < BH_WAVE; off <<= 1) {
+      const float f_before = __shfl_up(sum_f, off, BH_WAVE), i_before = __shfl_up(top_i, off, BH_WAVE);
+      if (lane >= off) {
+        top_i = fmaxf(i_before + sum_f, top_i);
+        sum_f = f_before + sum_f;
       }
-      m = next;
     }
+    const float mine = fmaxf(m + sum_f, top_i);
+    float before = __shfl_up(mine, 1, BH_WAVE);
+    if (lane == 0) before = m;
     if (t < rows) {
       float* out = beside + ((size_t)(row0 + t) * H + head) * ML_BESIDE;
       out[0] = expf(gate_f + before - mine);
       out[1] = expf(gate_i - mine);
       out[2] = mine;
     }
+    m = __shfl(mine, BH_WAVE - 1, BH_WAVE);
   }
   if (lane == 0 && rows > 0) *m_at = m;
 }
@@ -68,12 +71,34 @@ extern "C" int bh_mlstm_gates(const float* pre, const float* bias, float cap, fl
 }
 
 // ---- the recurrence --------------------------------------------------------------------------------------------
-// A workgroup a (sequence, head, tile of 16 columns).  Thread (column c, slice s) keeps rows s, s + 16, ... of column c in
-// registers; the 16 slices of a column are neighbouring lanes, so a row's read-out is added up inside the wave.  16 rows of q, k,
-// the tile's values and the gates' factors go through LDS at a time, the next 16 asked for before these are walked.
+// A workgroup a (sequence, head, tile of 16 columns).  Thread (column c, slice s) keeps rows s R .. s R + R - 1 of column c in
+// registers; the 16 slices of a column are neighbouring lanes.  16 rows of q, k (times b_t), the tile's values and the a_t go
+// through LDS at a time, the next 16 asked for before these are walked (two stages in flight brought nothing and cost 70
+// registers).  The walk over a stage's rows is unrolled and keeps
+// every row's share of the read-out in a register; the 16 shares of 16 lanes are then added up crosswise in 15 exchanges
+// (each lane ends with one row's sum, always in the same order), so no row waits for an exchange.
 #define ML_COLS 16
 #define ML_SLICES 16
 #define ML_STAGE 16
+
+// x of another lane of the same row of 16 lanes, by a data-parallel move: CTRL 0x140 the row mirrored (lane ^ 15), 0x141 its
+// halves mirrored (lane ^ 7), 0x1B quads reversed (lane ^ 3), 0xB1 neighbours swapped (lane ^ 1).
+template <int CTRL>
+__device__ inline float lanes_moved(float x) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, false));
+}
+
+// One exchange of the crosswise sum: acc[0 .. 2 SPAN) are the shares of 2 SPAN rows; the lane keeps the SPAN rows whose bit
+// SPAN is its own, adds what its partner (CTRL) held of them, and leaves them in acc[0 .. SPAN).
+template <int SPAN, int CTRL>
+__device__ inline void hand_over(float (&acc)[ML_STAGE], int lane) {
+  const bool upper = (lane & SPAN) != 0;
+#pragma unroll
+  for (int i = 0; i < SPAN; ++i) {
+    const float give = upper ? acc[i] : acc[i + SPAN], keep = upper ? acc[i + SPAN] : acc[i];
+    acc[i] = keep + lanes_moved<CTRL>(give);
+  }
+}
 
 template <typename T, int R>
 __global__ __launch_bounds__(ML_COLS * ML_SLICES) void mlstm_scan_kernel(
@@ -81,8 +106,8 @@ __global__ __launch_bounds__(ML_COLS * ML_SLICES) void mlstm_scan_kernel(
     float* __restrict__ state, long slot_stride, const int32_t* __restrict__ seq_start, const int32_t* __restrict__ seq_slot,
     float* __restrict__ read, float* beside, int H, int dim, int vdim, int tiles, float q_scale) {
   constexpr int DIM = ML_SLICES * R;      // the rows of a column that the registers hold (dim <= DIM)
-  __shared__ float s_q[ML_STAGE][DIM];
-  __shared__ float s_k[ML_STAGE][DIM];    // times b_t already
+  __shared__ __attribute__((aligned(16))) float s_q[ML_STAGE][DIM];
+  __shared__ __attribute__((aligned(16))) float s_k[ML_STAGE][DIM];    // times b_t already
   __shared__ float s_v[ML_STAGE][ML_COLS];
   __shared__ float s_a[ML_STAGE];
   const int tile = blockIdx.x % tiles, unit = blockIdx.x / tiles;
@@ -96,10 +121,10 @@ __global__ __launch_bounds__(ML_COLS * ML_SLICES) void mlstm_scan_kernel(
   float S[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) {
-    const int d = s + ML_SLICES * r;
+    const int d = s * R + r;
     S[r] = (column <= vdim && d < dim) ? mine[d] : 0.f;
   }
-  // what this thread brings into a stage: row `c` of it, dimensions s + 16 r of q and k; the tile's value (c, s as row, column)
+  // what this thread brings into a stage: row `c` of it, dimensions s R + r of q and k; the tile's value (c, s as row, column)
   float next_q[R], next_k[R], next_v = 0.f, next_a = 1.f, next_b = 0.f;
   auto ask = [&](int base) {
     const int t = base + c;
@@ -107,7 +132,7 @@ __global__ __launch_bounds__(ML_COLS * ML_SLICES) void mlstm_scan_kernel(
     const T* x = proj + (size_t)(row0 + (live ? t : 0)) * row_stride + (size_t)head * dim;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      const int d = s + ML_SLICES * r;
+      const int d = s * R + r;
       const bool there = live && d < dim;
       next_q[r] = there ? to_f32(x[q_off + d]) : 0.f;
       next_k[r] = there ? to_f32(x[k_off + d]) : 0.f;
@@ -125,37 +150,44 @@ __global__ __launch_bounds__(ML_COLS * ML_SLICES) void mlstm_scan_kernel(
     __syncthreads();      // the stage before has been walked by all
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      s_q[c][s + ML_SLICES * r] = next_q[r] * q_scale;
-      s_k[c][s + ML_SLICES * r] = next_k[r] * next_b;
+      s_q[c][s * R + r] = next_q[r] * q_scale;
+      s_k[c][s * R + r] = next_k[r] * next_b;
     }
     s_v[c][s] = next_v;
     if (s == 0) s_a[c] = next_a;
     __syncthreads();
     if (base + ML_STAGE < rows) ask(base + ML_STAGE);
-    const int live = rows - base < ML_STAGE ? rows - base : ML_STAGE;
-    for (int t = 0; t < live; ++t) {
+    // (rows beyond the end stand in LDS as a = 1, k = 0: they change nothing and their sums are not stored)
+    float acc[ML_STAGE];
+#pragma unroll
+    for (int t = 0; t < ML_STAGE; ++t) {
       const float a = s_a[t], v = s_v[t][c];
-      float acc = 0.f;
+      float sum = 0.f;
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        const int d = s + ML_SLICES * r;
-        S[r] = fmaf(a, S[r], s_k[t][d] * v);
-        acc = fmaf(S[r], s_q[t][d], acc);
+        S[r] = fmaf(a, S[r], s_k[t][s * R + r] * v);
+        sum = fmaf(S[r], s_q[t][s * R + r], sum);
       }
-      acc += __shfl_xor(acc, 8, BH_WAVE);
-      acc += __shfl_xor(acc, 4, BH_WAVE);
-      acc += __shfl_xor(acc, 2, BH_WAVE);
-      acc += __shfl_xor(acc, 1, BH_WAVE);
-      if (s == 0) {
-        const size_t row = (size_t)(row0 + base + t);
-        if (column < vdim) read[row * H * vdim + (size_t)head * vdim + column] = acc;
-        else if (column == vdim) beside[(row * H + head) * ML_BESIDE + 3] = acc;
-      }
+      acc[t] = sum;
+    }
+    // Lane s of a column's 16 ends with row s's sum.  Four exchanges with the lane whose number differs in all four bits, in
+    // the lower three, two and one (a row of 16 lanes mirrored, its halves mirrored, quads reversed, neighbours swapped: the
+    // data-parallel moves of the vector unit): each time a lane keeps the rows whose bit is its own and hands over the
+    // others' shares.  (Written out by templates: a loop over the spans is not unrolled, its registers are then found by
+    // number at run time, and that took more time than everything else in this kernel.)
+    hand_over<8, 0x140>(acc, s);
+    hand_over<4, 0x141>(acc, s);
+    hand_over<2, 0x1B>(acc, s);
+    hand_over<1, 0xB1>(acc, s);
+    if (base + s < rows) {
+      const size_t row = (size_t)(row0 + base + s);
+      if (column < vdim) read[row * H * vdim + (size_t)head * vdim + column] = acc[0];
+      else if (column == vdim) beside[(row * H + head) * ML_BESIDE + 3] = acc[0];
     }
   }
 #pragma unroll
   for (int r = 0; r < R; ++r) {
-    const int d = s + ML_SLICES * r;
+    const int d = s * R + r;
     if (column <= vdim && d < dim) mine[d] = S[r];
   }
 }
