@@ -69,6 +69,9 @@ def parse():
                              "layers that run another layer's tensors) at layer sizes of real models beside Pudorax and Qwen3 at "
                              "equal width and as many layer runs: prefill and decode tokens per second, and every kernel of the "
                              "new design beside its like with the fraction of its roofline; prints one JSON line and exits")
+    parser.add_argument("--alone", action="store_true",
+                        help="with --dupidra: the new design's two models only, without the models beside them and without the "
+                             "kernels timed alone (what a profiler should see of it)")
     parser.add_argument("--sampling", action="store_true",
                         help="time the selection kernel on 1, 8 and 64 rows of 151,936 logits (greedy, at a temperature, with "
                              "top-k, with top-p on rows of three spreads, with both), print the microseconds and exit")
@@ -787,6 +790,8 @@ def dupidra_bench(args, torch):
                 "qwen3": dict(QWEN3_8B, num_hidden_layers=8, hidden_size=width, num_attention_heads=heads,
                               num_key_value_heads=heads // 4, intermediate_size=3 * width, vocab_size=32768)}
         point = {"width": width, "heads": heads, "layer_runs": 8}
+        if args.alone:
+            trio = {"dupidra": trio["dupidra"]}
         for name, config in trio.items():
             model = random_model_on_device(config, seed=0, dtype="bfloat16", device=device)
             engine = Engine(model=model, dtype="bfloat16", max_tokens=args.batch * (-(-args.context // 64) * 64),
@@ -804,7 +809,7 @@ def dupidra_bench(args, torch):
     line = {"metric": f"Dupidra beside Pudorax and Qwen3 at equal width and as many layer runs: decode tok/s @ batch {args.batch}, context {args.context}; prefill of {t} tokens",
             "unit": "tok/s", "value": points[-1]["dupidra"]["decode_tok_per_s"], "dtype": "bf16", "data": "synthetic", "n_gpus": 1,
             "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "points": points,
-            "kernels": dupidra_kernels(kernels, torch, 4096, 32, args.context)}
+            "kernels": {} if args.alone else dupidra_kernels(kernels, torch, 4096, 32, args.context)}
     print(json.dumps(line))
     return 0
 

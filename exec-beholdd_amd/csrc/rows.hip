@@ -78,6 +78,56 @@ __global__ __launch_bounds__(256) void sum_layernorm_kernel(float* __restrict__ 
   }
 }
 
+// The same for rows of up to 256 * PER elements: a thread keeps its PER elements of the sum in registers, so the row is read
+// once and written once and nothing waits for its own stores (a step of few rows is three trips to memory shorter).
+template <typename TO, int PER>
+__global__ __launch_bounds__(256) void sum_layernorm_held_kernel(float* __restrict__ h, const float* __restrict__ y, float alpha,
+                                                                 const float* __restrict__ w, const float* __restrict__ b,
+                                                                 TO* __restrict__ rounded, int width, float eps, int out_block_rows) {
+  __shared__ float scratch[8];
+  const int r = blockIdx.x;
+  float* row = h + (size_t)r * width;
+  const float* add = y + (size_t)r * width;
+  float held[PER];
+  float sum = 0.f;
+#pragma unroll
+  for (int k = 0; k < PER; ++k) {
+    const int i = threadIdx.x + k * 256;
+    held[k] = i < width ? fmaf(alpha, row[i], add[i]) : 0.f;
+    sum += held[k];
+  }
+  const float mean = block_sum(sum, scratch) / (float)width;
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < PER; ++k) {
+    const float d = threadIdx.x + k * 256 < width ? held[k] - mean : 0.f;
+    ss += d * d;
+  }
+  const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / (float)width + eps);
+#pragma unroll
+  for (int k = 0; k < PER; ++k) {
+    const int i = threadIdx.x + k * 256;
+    if (i < width) {
+      const float v = (held[k] - mean) * inv * w[i] + (b ? b[i] : 0.f);
+      row[i] = v;
+      if (rounded) rounded[bh_rows_index(out_block_rows, r, i, width)] = from_f32<TO>(v);
+    }
+  }
+}
+
+template <typename TO>
+static void sum_layernorm_launch(float* h, const float* y, float alpha, const float* w, const float* b, TO* rounded, int n_rows,
+                                 int width, float eps, int out_block_rows, hipStream_t stream) {
+  if (width <= 256 * 4)
+    sum_layernorm_held_kernel<TO, 4><<<n_rows, 256, 0, stream>>>(h, y, alpha, w, b, rounded, width, eps, out_block_rows);
+  else if (width <= 256 * 16)
+    sum_layernorm_held_kernel<TO, 16><<<n_rows, 256, 0, stream>>>(h, y, alpha, w, b, rounded, width, eps, out_block_rows);
+  else if (width <= 256 * 32)
+    sum_layernorm_held_kernel<TO, 32><<<n_rows, 256, 0, stream>>>(h, y, alpha, w, b, rounded, width, eps, out_block_rows);
+  else
+    sum_layernorm_kernel<TO><<<n_rows, 256, 0, stream>>>(h, y, alpha, w, b, rounded, width, eps, out_block_rows);
+}
+
 extern "C" int bh_sum_layernorm(float* h, const float* y, float alpha, const float* w, const float* b, void* rounded,
                                 int out_dtype, int n_rows, int width, float eps, int out_block_rows, hipStream_t stream) {
   BH_REQUIRE(n_rows > 0 && width > 0, "sum_layernorm: sizes must be positive");
@@ -85,9 +135,9 @@ extern "C" int bh_sum_layernorm(float* h, const float* y, float alpha, const flo
   BH_REQUIRE(out_block_rows == 0 || (rounded && (out_block_rows == 8 || out_block_rows == 16) && width % 32 == 0 && out_dtype == BH_BF16),
              "sum_layernorm: rows in blocks of %d of width %d are not written", out_block_rows, width);
   if (rounded == nullptr || out_dtype == BH_F32)
-    sum_layernorm_kernel<float><<<n_rows, 256, 0, stream>>>(h, y, alpha, w, b, (float*)rounded, width, eps, out_block_rows);
+    sum_layernorm_launch<float>(h, y, alpha, w, b, (float*)rounded, n_rows, width, eps, out_block_rows, stream);
   else if (out_dtype == BH_BF16)
-    sum_layernorm_kernel<bf16_t><<<n_rows, 256, 0, stream>>>(h, y, alpha, w, b, (bf16_t*)rounded, width, eps, out_block_rows);
+    sum_layernorm_launch<bf16_t>(h, y, alpha, w, b, (bf16_t*)rounded, n_rows, width, eps, out_block_rows, stream);
   else
     return bh_fail("sum_layernorm: unknown dtype %d", out_dtype);
   return bh_check_launch("sum_layernorm");
