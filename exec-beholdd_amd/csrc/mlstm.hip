@@ -159,14 +159,17 @@ __global__ __launch_bounds__(ML_COLS * ML_SLICES) void mlstm_scan_kernel(
     if (base + ML_STAGE < rows) ask(base + ML_STAGE);
     // (rows beyond the end stand in LDS as a = 1, k = 0: they change nothing and their sums are not stored)
     float acc[ML_STAGE];
+    const int live = rows - base < ML_STAGE ? rows - base : ML_STAGE;      // (a decode step walks one row, not sixteen)
 #pragma unroll
     for (int t = 0; t < ML_STAGE; ++t) {
-      const float a = s_a[t], v = s_v[t][c];
       float sum = 0.f;
+      if (t < live) {
+        const float a = s_a[t], v = s_v[t][c];
 #pragma unroll
-      for (int r = 0; r < R; ++r) {
-        S[r] = fmaf(a, S[r], s_k[t][s * R + r] * v);
-        sum = fmaf(S[r], s_q[t][s * R + r], sum);
+        for (int r = 0; r < R; ++r) {
+          S[r] = fmaf(a, S[r], s_k[t][s * R + r] * v);
+          sum = fmaf(S[r], s_q[t][s * R + r], sum);
+        }
       }
       acc[t] = sum;
     }

@@ -78,13 +78,13 @@ __global__ __launch_bounds__(256) void sum_layernorm_kernel(float* __restrict__ 
   }
 }
 
-// The same for rows of up to 256 * PER elements: a thread keeps its PER elements of the sum in registers, so the row is read
+// The same for rows of up to THREADS * PER elements: a thread keeps its PER elements of the sum in registers, so the row is read
 // once and written once and nothing waits for its own stores (a step of few rows is three trips to memory shorter).
-template <typename TO, int PER>
-__global__ __launch_bounds__(256) void sum_layernorm_held_kernel(float* __restrict__ h, const float* __restrict__ y, float alpha,
+template <typename TO, int PER, int THREADS>
+__global__ __launch_bounds__(THREADS) void sum_layernorm_held_kernel(float* __restrict__ h, const float* __restrict__ y, float alpha,
                                                                  const float* __restrict__ w, const float* __restrict__ b,
                                                                  TO* __restrict__ rounded, int width, float eps, int out_block_rows) {
-  __shared__ float scratch[8];
+  __shared__ float scratch[THREADS / BH_WAVE];
   const int r = blockIdx.x;
   float* row = h + (size_t)r * width;
   const float* add = y + (size_t)r * width;
@@ -92,7 +92,7 @@ __global__ __launch_bounds__(256) void sum_layernorm_held_kernel(float* __restri
   float sum = 0.f;
 #pragma unroll
   for (int k = 0; k < PER; ++k) {
-    const int i = threadIdx.x + k * 256;
+    const int i = threadIdx.x + k * THREADS;
     held[k] = i < width ? fmaf(alpha, row[i], add[i]) : 0.f;
     sum += held[k];
   }
@@ -100,13 +100,13 @@ __global__ __launch_bounds__(256) void sum_layernorm_held_kernel(float* __restri
   float ss = 0.f;
 #pragma unroll
   for (int k = 0; k < PER; ++k) {
-    const float d = threadIdx.x + k * 256 < width ? held[k] - mean : 0.f;
+    const float d = threadIdx.x + k * THREADS < width ? held[k] - mean : 0.f;
     ss += d * d;
   }
   const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / (float)width + eps);
 #pragma unroll
   for (int k = 0; k < PER; ++k) {
-    const int i = threadIdx.x + k * 256;
+    const int i = threadIdx.x + k * THREADS;
     if (i < width) {
       const float v = (held[k] - mean) * inv * w[i] + (b ? b[i] : 0.f);
       row[i] = v;
@@ -118,14 +118,21 @@ __global__ __launch_bounds__(256) void sum_layernorm_held_kernel(float* __restri
 template <typename TO>
 static void sum_layernorm_launch(float* h, const float* y, float alpha, const float* w, const float* b, TO* rounded, int n_rows,
                                  int width, float eps, int out_block_rows, hipStream_t stream) {
-  if (width <= 256 * 4)
-    sum_layernorm_held_kernel<TO, 4><<<n_rows, 256, 0, stream>>>(h, y, alpha, w, b, rounded, width, eps, out_block_rows);
-  else if (width <= 256 * 16)
-    sum_layernorm_held_kernel<TO, 16><<<n_rows, 256, 0, stream>>>(h, y, alpha, w, b, rounded, width, eps, out_block_rows);
-  else if (width <= 256 * 32)
-    sum_layernorm_held_kernel<TO, 32><<<n_rows, 256, 0, stream>>>(h, y, alpha, w, b, rounded, width, eps, out_block_rows);
-  else
+#define BH_SL(PER, THREADS) \
+  sum_layernorm_held_kernel<TO, PER, THREADS><<<n_rows, THREADS, 0, stream>>>(h, y, alpha, w, b, rounded, width, eps, out_block_rows)
+  if (n_rows <= 64 && width > 1024 && width <= 1024 * 8) {      // few rows: a row on sixteen waves, a few elements a thread
+    if (width <= 1024 * 4) BH_SL(4, 1024);
+    else BH_SL(8, 1024);
+  } else if (width <= 256 * 4) {
+    BH_SL(4, 256);
+  } else if (width <= 256 * 16) {
+    BH_SL(16, 256);
+  } else if (width <= 256 * 32) {
+    BH_SL(32, 256);
+  } else {
     sum_layernorm_kernel<TO><<<n_rows, 256, 0, stream>>>(h, y, alpha, w, b, rounded, width, eps, out_block_rows);
+  }
+#undef BH_SL
 }
 
 extern "C" int bh_sum_layernorm(float* h, const float* y, float alpha, const float* w, const float* b, void* rounded,
