@@ -74,7 +74,8 @@ extern "C" int bh_mlstm_gates(const float* pre, const float* bias, float cap, fl
 // A workgroup a (sequence, head, tile of 16 columns).  Thread (column c, slice s) keeps rows s R .. s R + R - 1 of column c in
 // registers; the 16 slices of a column are neighbouring lanes.  16 rows of q, k (times b_t), the tile's values and the a_t go
 // through LDS at a time, the next 16 asked for before these are walked (two stages in flight brought nothing and cost 70
-// registers).  The walk over a stage's rows is unrolled and keeps
+// registers; a stage that asks every row whether it is there, so that a decode step walks one row and not sixteen, was
+// slower on prompts and no faster in decode steps).  The walk over a stage's rows is unrolled and keeps
 // every row's share of the read-out in a register; the 16 shares of 16 lanes are then added up crosswise in 15 exchanges
 // (each lane ends with one row's sum, always in the same order), so no row waits for an exchange.
 #define ML_COLS 16
@@ -159,17 +160,14 @@ __global__ __launch_bounds__(ML_COLS * ML_SLICES) void mlstm_scan_kernel(
     if (base + ML_STAGE < rows) ask(base + ML_STAGE);
     // (rows beyond the end stand in LDS as a = 1, k = 0: they change nothing and their sums are not stored)
     float acc[ML_STAGE];
-    const int live = rows - base < ML_STAGE ? rows - base : ML_STAGE;      // (a decode step walks one row, not sixteen)
 #pragma unroll
     for (int t = 0; t < ML_STAGE; ++t) {
+      const float a = s_a[t], v = s_v[t][c];
       float sum = 0.f;
-      if (t < live) {
-        const float a = s_a[t], v = s_v[t][c];
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-          S[r] = fmaf(a, S[r], s_k[t][s * R + r] * v);
-          sum = fmaf(S[r], s_q[t][s * R + r], sum);
-        }
+      for (int r = 0; r < R; ++r) {
+        S[r] = fmaf(a, S[r], s_k[t][s * R + r] * v);
+        sum = fmaf(S[r], s_q[t][s * R + r], sum);
       }
       acc[t] = sum;
     }

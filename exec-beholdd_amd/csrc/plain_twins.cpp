@@ -141,7 +141,7 @@ int bhp_qk_norm_rope_cache(const void* qkv, int dtype, void* q_out, const void* 
   return 0;
 }
 
-// out[row, head] = softmax(q . K * scale) V over the keys max(0, p - window + 1) .. p of the row's sequence
+// out[row, head] = softmax(q . K * scale) V over the keys bh_first_visible(p, window) .. p of the row's sequence (layout.h)
 // (generic.hip: bh_attention_generic; attention_bf16.hip and attention_prefill_bf16.hip for bfloat16;
 // crates/beholdd-backend/src/cpu.rs:693-837: dots and value sums in double, softmax in float32)
 int bhp_attention(const void* q, void* out, int dtype, const void* k_pages, const void* v_pages,

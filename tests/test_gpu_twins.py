@@ -102,7 +102,10 @@ class Layout:
 
 @pytest.mark.parametrize("dtype,code,head_dim,rot,window", [(torch.float32, F32, 48, 48, 0), (torch.float32, F32, 80, 32, 70),
                                                             (torch.bfloat16, BF16, 64, 64, 0), (torch.bfloat16, BF16, 128, 128, 100),
-                                                            (torch.bfloat16, BF16, 48, 0, 0)])
+                                                            (torch.bfloat16, BF16, 48, 0, 0),
+                                                            # (a negative number: chunks of that many positions, counted from 0)
+                                                            (torch.float32, F32, 48, 48, -40), (torch.bfloat16, BF16, 64, 64, -64),
+                                                            (torch.bfloat16, BF16, 128, 128, -33)])
 def test_cache_write_and_attention_and_their_twins(K, twins, dtype, code, head_dim, rot, window):
     """Sequences with pasts of 0, 70 and 5 tokens get 9, 1 and 130 more rows in one step: the writing kernel fills
     the same places of the same pages as its twin, and the attention kernel (the generic one, or the matrix-core
@@ -155,7 +158,7 @@ def test_cache_write_and_attention_and_their_twins(K, twins, dtype, code, head_d
     out = torch.empty_like(q_dev)
     layout = Layout(dev(np.asarray(starts, np.int32)), 3, max(new for _, new in lengths), max(positions))
     K.attention(q_dev, out, k_dev, v_dev, dev(table), dev(np.asarray(row_seq, np.int32)), dev(np.asarray(positions, np.int32)),
-                n_heads, kv_heads, head_dim, scale, window, layout=layout)
+                n_heads, kv_heads, head_dim, scale, max(window, 0), layout=layout, chunk=max(-window, 0))
     want = twins.attention(host(q_dev), k_twin, v_twin, table, row_seq, positions, n_heads, kv_heads, head_dim, scale, window, order, code)
     assert rel(host(out), want) < (1e-5 if code == F32 else 1.2e-2)
 
