@@ -96,12 +96,22 @@ DEEP = _with_borrowers({
                mlstm(4, 32, 32, 12.0, mlp=moe(8, 4, 32, 1.0)),
                attention(8, 2, 32, 32, 0.18, chunk=33, rot_dims=8, base=1000.0, mlp=dense(200))],
 }, [(3, 1), (4, 0), (5, 2), (6, 1)])
+# Sizes that are multiples of nothing: a width of 100, heads of 6, 10, 5 and 7 dimensions, a latent of 50, feed-forwards of 10
+# and 30, a vocabulary of 101, seven experts of which three are used; a borrower that stands ahead of its owner.
+ODD = {
+    "architecture": "Dupidra", "vocab": 101, "width": 100, "postln_alpha": 2.25, "norm": {"eps": 1e-4},
+    "layers": [attention(3, 1, 6, 10, 0.4, chunk=37, rot_dims=2, base=300.0, mlp=moe(7, 3, 10, 0.9)),
+               latent(5, 10, 6, 50, 0.3, window=45, mlp=dense(30)),
+               mlstm(3, 5, 7, 4.0, mlp=moe(3, 2, 18, 2.0))],
+}
+ODD["layers"].insert(0, borrowed(ODD["layers"], 0, 2))      # runs the memory's tensors, which are then layer 3's
+ODD["layers"][0]["weights_of"] = 3
 # The same layers with a residual that weighs little beside the sublayers (with matrices of twice the usual size): the
 # logits come from the embedding table too, so a model whose residual dominates predicts its last token over and over,
 # and greedy continuations would say nothing.
 GENERATING = dict(json.loads(json.dumps(MIXED)), postln_alpha=0.4)
 GENERATING_GAIN = 2.0
-CONFIGS = {"mixed": MIXED, "plain": PLAIN, "edges": EDGES, "deep": DEEP}
+CONFIGS = {"mixed": MIXED, "plain": PLAIN, "edges": EDGES, "deep": DEEP, "odd": ODD}
 
 
 def tensor_shapes(config):

@@ -191,7 +191,7 @@ def test_the_norm_stands_behind_the_weighted_sum():
 
 # ---- the engine's logic on the torch double -------------------------------------------------------------------
 
-LENGTHS = {"mixed": [5, 11, 1, 70, 33, 130], "plain": [1, 7, 23, 64, 90], "edges": [3, 65, 130, 2, 31], "deep": [2, 50, 129]}
+LENGTHS = {"mixed": [5, 11, 1, 70, 33, 130], "plain": [1, 7, 23, 64, 90], "edges": [3, 65, 130, 2, 31], "deep": [2, 50, 129], "odd": [1, 40, 100]}
 
 
 @pytest.mark.parametrize("name", sorted(LENGTHS))

@@ -62,7 +62,7 @@ def test_gelu(K, dtype):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("heads,kv_heads,dim,vdim,pad,turned,base,chunk", [
     (6, 2, 24, 40, 64, 8, 1e4, 20), (4, 4, 64, 64, 64, 64, 500.0, 64), (8, 1, 12, 20, 32, 0, 1.0, 1), (2, 2, 272, 16, 272, 64, 1e6, 100),
-    (3, 1, 128, 128, 128, 32, 1e6, 0), (16, 1, 64, 32, 64, 64, 5e4, 65), (17, 1, 32, 32, 32, 16, 1e4, 130)])
+    (3, 1, 128, 128, 128, 32, 1e6, 0), (16, 1, 64, 48, 64, 64, 2e4, 65), (17, 1, 32, 32, 32, 16, 1e4, 130)])
 def test_bias_head_norms_rotation_cache_write_and_chunked_attention(K, dtype, heads, kv_heads, dim, vdim, pad, turned, base, chunk):
     """From the projected rows to the attended heads: biases, every head normed with the one weight, rotation in halves, keys
     and values of different sizes through one padded head, chunks counted from position 0; a prompt in two portions that end
@@ -123,7 +123,7 @@ def test_heads_without_norm_bias_or_rotation_pass_as_they_are(K, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("heads,dim,vdim,rank,window", [(3, 16, 12, 32, 27), (8, 32, 32, 96, 64), (2, 8, 8, 20, 1), (5, 16, 16, 64, 65), (1, 32, 32, 32, 0)])
+@pytest.mark.parametrize("heads,dim,vdim,rank,window", [(3, 16, 12, 32, 27), (6, 32, 40, 96, 64), (2, 8, 8, 20, 1), (5, 16, 16, 64, 65), (1, 32, 32, 32, 0)])
 def test_windowed_attention_over_a_latent_without_a_rotated_part(K, dtype, heads, dim, vdim, rank, window):
     rng = np.random.default_rng(rank + window)
     t_len, eps, scale = 150, 1e-5, 0.25
@@ -162,7 +162,7 @@ def test_windowed_attention_over_a_latent_without_a_rotated_part(K, dtype, heads
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("heads,dim,vdim,cap,lengths", [(3, 8, 20, 9.0, [5, 1, 31]), (1, 16, 16, 1.0, [70]), (4, 32, 48, 12.0, [3, 17, 2]),
+@pytest.mark.parametrize("heads,dim,vdim,cap,lengths", [(3, 8, 20, 9.0, [5, 1, 31]), (1, 16, 16, 1.0, [70]), (4, 32, 40, 11.0, [3, 17, 2]),
                                                         (2, 80, 70, 15.0, [40]), (5, 4, 15, 8.0, [1, 1, 1, 1]), (2, 128, 128, 12.0, [9, 33]),
                                                         (1, 260, 16, 12.0, [18]), (3, 12, 33, 6.0, [200, 64, 65])])
 def test_matrix_memory(K, dtype, heads, dim, vdim, cap, lengths):
@@ -223,7 +223,7 @@ def folders(tmp_path_factory):
     return get
 
 
-LENGTHS = {"mixed": [5, 11, 1, 70, 33, 128, 300], "plain": [1, 7, 23, 64, 90, 200], "edges": [3, 65, 130, 2, 31, 330], "deep": [2, 50, 129, 260]}
+LENGTHS = {"mixed": [5, 11, 1, 70, 33, 128, 300], "plain": [1, 7, 23, 64, 90, 200], "edges": [3, 65, 130, 2, 31, 330], "deep": [2, 50, 129, 260], "odd": [1, 40, 100, 210]}
 
 
 @pytest.fixture(scope="module")
