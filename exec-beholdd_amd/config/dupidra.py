@@ -140,9 +140,10 @@ class DupidraConfig:
                 owner = layers[owner].weights_of
             if owner != index:
                 theirs = layers[owner]
-                if (theirs.kind, theirs.mixer, theirs.mlp) != (layer.kind, layer.mixer, layer.mlp):
+                # (the feed-forward is the owner's too: an entry that leaves it out runs the owner's, one that names another is wrong)
+                if (theirs.kind, theirs.mixer) != (layer.kind, layer.mixer) or (layer.mlp is not None and layer.mlp != theirs.mlp):
                     raise ConfigError(f"{origin}: layers[{index}] runs the tensors of layers[{owner}] but has other sizes")
-                layers[index] = DupidraLayer(layer.kind, layer.mixer, layer.mlp, owner)
+                layers[index] = DupidraLayer(theirs.kind, theirs.mixer, theirs.mlp, owner)
         return cls(architecture=architecture, vocab=vocab, hidden=hidden, layers=tuple(layers), rms_eps=rms_eps, postln_alpha=alpha)
 
     @staticmethod

@@ -46,6 +46,9 @@ def test_a_borrowing_layer_runs_its_owners_parts_with_memory_of_its_own():
     model = beholdd.registry.resolve_architecture(dm.MIXED).build(config)
     needs = model.entry_needs
     assert len(needs) == 7 and needs[4] == needs[1] and needs[5] == needs[0] and needs[6] == needs[2]
+    bare = copy.deepcopy(dm.MIXED)
+    bare["layers"][4].pop("mlp")                                            # the feed-forward is the owner's, named again or not
+    assert DupidraConfig.from_dict(bare).layers[4].mlp == config.layers[1].mlp
     chained = copy.deepcopy(dm.MIXED)
     chained["layers"].append(dm.borrowed(chained["layers"], 7, 4))          # borrows from a borrower: runs the first owner's
     assert DupidraConfig.from_dict(chained).schedule()[-1] == (1, 7)
