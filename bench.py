@@ -759,6 +759,10 @@ def dupidra_kernels(K, torch, width, heads, context, rank=256):
         m_weight = torch.ones(heads * vdim, device=dev)
         us = timed(lambda: K.mlstm_finish(read, beside, m_proj, 2 * heads * m_dim + heads * vdim, m_weight, 1e-6, m_out, heads, vdim), torch)
         note(f"mlstm_finish, {tag}", us, read.numel() * 4 + 2 * m_out.numel() * 2)
+        if each == 1:      # the three in one launch, as a decode step runs them
+            us = timed(lambda: K.mlstm_step(m_proj, 0, heads * m_dim, 2 * heads * m_dim, 2 * heads * m_dim + heads * vdim, pre, gate_bias, 15.0,
+                                            m_state, slots, m_weight, 1e-6, m_out, heads, m_dim, vdim), torch)
+            note(f"mlstm_step (gates, scan and finish in one launch), {tag}", us, 2 * m_state.numel() * 4 + m_proj.numel() * 2 + m_out.numel() * 2)
         l_proj = torch.randn(rows, 4 * heads * dim, device=dev).to(bf16)
         l_state = torch.zeros(seqs, heads, dim, vdim, device=dev)
         decay = torch.full((heads,), 0.99, device=dev)

@@ -9,6 +9,7 @@
 //   mlstm_gates    a_t, b_t and m_t of every row and head, the rows of a sequence in order from the slot's m, which it moves on
 //   mlstm_scan     the recurrence over the columns: S^T q and n . q of every row and head, from the slot's state, which it moves on
 //   mlstm_finish   the division, the heads' RMS norm (no mean taken off), the weight and the sigmoid gate, for the output projection
+//   mlstm_step     all three for a step of one row a sequence (a decode step), one launch
 // Everything here is float32 but the projected q, k, v and the gate's pre-activation, which come in the activation type.
 #include "common.h"
 
@@ -274,4 +275,115 @@ extern "C" int bh_mlstm_finish(const float* read, const float* beside, const voi
   else
     return bh_fail("mlstm_finish: unknown dtype %d", dtype);
   return bh_check_launch("mlstm_finish");
+}
+
+// ---- a decode step: gates, one step of the recurrence and the read-out in one launch ------------------------------------
+// A workgroup a (sequence, head); the sequence brings one row.  Every thread makes the gates' numbers for itself (a handful of
+// operations), q and b k stand in LDS, the columns are walked 16 at a time by the scan's threads (column c, slice s), each
+// column's read-out is added up across its 16 lanes and left in LDS, and the workgroup then divides, norms and gates its head.
+template <typename T, int R>
+__global__ __launch_bounds__(ML_COLS * ML_SLICES) void mlstm_step_kernel(
+    const T* __restrict__ proj, int row_stride, int q_off, int k_off, int v_off, int g_off, const float* __restrict__ pre,
+    const float* __restrict__ bias, float cap, float* __restrict__ state, long slot_stride, const int32_t* __restrict__ seq_slot,
+    const float* __restrict__ w, float eps, T* __restrict__ out, int H, int dim, int vdim, float q_scale, int out_block_rows) {
+  constexpr int DIM = ML_SLICES * R;
+  extern __shared__ float s_o[];      // vdim + 1 read-outs: the values' columns, then n . q
+  __shared__ float s_q[DIM];
+  __shared__ float s_k[DIM];
+  __shared__ float scratch[ML_COLS * ML_SLICES / BH_WAVE];
+  const int seq = blockIdx.x / H, head = blockIdx.x % H, row = seq;
+  const int tid = threadIdx.x, c = tid / ML_SLICES, s = tid % ML_SLICES;
+  const int head_floats = (vdim + 1) * dim + 1;
+  float* held = state + (size_t)seq_slot[seq] * slot_stride + (size_t)head * head_floats;
+  const T* x = proj + (size_t)row * row_stride;
+  // the gates (mlstm_gates_kernel's numbers for one row)
+  const float inv_cap = 1.0f / cap;
+  const float* gate_in = pre + (size_t)row * 2 * H;
+  const float gate_i = cap * tanhf((gate_in[head] + (bias ? bias[head] : 0.f)) * inv_cap);
+  const float z = cap * tanhf((gate_in[H + head] + (bias ? bias[H + head] : 0.f)) * inv_cap);
+  const float gate_f = fminf(z, 0.f) - log1pf(expf(-fabsf(z)));
+  const float m_before = held[head_floats - 1];
+  const float m = fmaxf(gate_f + m_before, gate_i);
+  const float a = expf(gate_f + m_before - m), b = expf(gate_i - m);
+  for (int d = tid; d < DIM; d += blockDim.x) {
+    s_q[d] = d < dim ? to_f32(x[q_off + head * dim + d]) * q_scale : 0.f;
+    s_k[d] = d < dim ? to_f32(x[k_off + head * dim + d]) * b : 0.f;
+  }
+  __syncthreads();
+  for (int first = 0; first <= vdim; first += ML_COLS) {
+    const int column = first + c;
+    float* mine = held + (size_t)column * dim;
+    const float v = column < vdim ? to_f32(x[v_off + head * vdim + column]) : 1.f;
+    float sum = 0.f;
+    if (column <= vdim) {
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const int d = s * R + r;
+        if (d < dim) {
+          const float now = fmaf(a, mine[d], s_k[d] * v);
+          mine[d] = now;
+          sum = fmaf(now, s_q[d], sum);
+        }
+      }
+    }
+    sum += lanes_moved<0x140>(sum);      // across the column's 16 lanes: every lane ends with the whole
+    sum += lanes_moved<0x141>(sum);
+    sum += lanes_moved<0x1B>(sum);
+    sum += lanes_moved<0xB1>(sum);
+    if (s == 0 && column <= vdim) s_o[column] = sum;
+  }
+  __syncthreads();
+  if (tid == 0) held[head_floats - 1] = m;
+  const float under = 1.0f / (fmaxf(fabsf(s_o[vdim]), expf(-m)) + 1e-6f);
+  float ss = 0.f;
+  for (int e = tid; e < vdim; e += blockDim.x) {
+    const float o = s_o[e] * under;
+    ss += o * o;
+  }
+  const float norm = 1.0f / sqrtf(block_sum(ss, scratch) / (float)vdim + eps);
+  for (int e = tid; e < vdim; e += blockDim.x) {
+    const int at = head * vdim + e;
+    const float g = to_f32(x[g_off + at]);
+    const float y = s_o[e] * under * norm * (w ? w[at] : 1.f) / (1.0f + expf(-g));
+    out[bh_rows_index(out_block_rows, row, at, H * vdim)] = from_f32<T>(y);
+  }
+}
+
+// A step in which sequence b brings the one row b: proj, pre, bias as for mlstm_gates and mlstm_scan, w and out as for
+// mlstm_finish; the slots' states are moved on.
+extern "C" int bh_mlstm_step(const void* proj, int dtype, int row_stride, int q_off, int k_off, int v_off, int g_off, const float* pre,
+                             const float* bias, float cap, float* state, long slot_stride, const int32_t* seq_slot, const float* w,
+                             float eps, void* out, int n_seqs, int H, int dim, int vdim, int out_block_rows, hipStream_t stream) {
+  BH_REQUIRE(n_seqs > 0 && H > 0 && dim > 0 && vdim > 0 && cap > 0.f, "mlstm_step: sizes and the cap must be positive");
+  BH_REQUIRE(dim <= ML_SLICES * 32, "mlstm_step: heads of %d key dimensions are above the limit of %d", dim, ML_SLICES * 32);
+  BH_REQUIRE((long)H * ((long)(vdim + 1) * dim + 1) <= slot_stride, "mlstm_step: %d heads of %d x %d do not fit a slot's %ld floats", H, dim,
+             vdim, slot_stride);
+  BH_REQUIRE(q_off >= 0 && k_off >= 0 && v_off >= 0 && g_off >= 0 && q_off + H * dim <= row_stride && k_off + H * dim <= row_stride &&
+                 v_off + H * vdim <= row_stride && g_off + H * vdim <= row_stride, "mlstm_step: q, k, v and the gate lie outside a row of %d", row_stride);
+  BH_REQUIRE(out_block_rows == 0 || ((out_block_rows == 8 || out_block_rows == 16) && (H * vdim) % 32 == 0 && dtype == BH_BF16),
+             "mlstm_step: rows in blocks of %d of width %d are not written", out_block_rows, H * vdim);
+  const size_t lds = (size_t)(vdim + 1) * sizeof(float);
+  BH_REQUIRE(lds <= 32 * 1024, "mlstm_step: heads of %d values do not fit the local memory", vdim);
+  BH_REQUIRE((long)n_seqs * H < (1L << 31), "mlstm_step: too many workgroups");
+  const float q_scale = 1.0f / sqrtf((float)dim);
+  const int per = (dim + ML_SLICES - 1) / ML_SLICES;
+#define BH_MS(T, R)                                                                                                                 \
+  mlstm_step_kernel<T, R><<<n_seqs * H, ML_COLS * ML_SLICES, lds, stream>>>((const T*)proj, row_stride, q_off, k_off, v_off, g_off, pre, \
+                                                                          bias, cap, state, slot_stride, seq_slot, w, eps, (T*)out, H, \
+                                                                          dim, vdim, q_scale, out_block_rows)
+#define BH_MS_SIZES(T)              \
+  do {                              \
+    if (per <= 1) BH_MS(T, 1);      \
+    else if (per <= 2) BH_MS(T, 2); \
+    else if (per <= 4) BH_MS(T, 4); \
+    else if (per <= 8) BH_MS(T, 8); \
+    else if (per <= 16) BH_MS(T, 16); \
+    else BH_MS(T, 32);              \
+  } while (0)
+  if (dtype == BH_F32) BH_MS_SIZES(float);
+  else if (dtype == BH_BF16) BH_MS_SIZES(bf16_t);
+  else return bh_fail("mlstm_step: unknown dtype %d", dtype);
+#undef BH_MS_SIZES
+#undef BH_MS
+  return bh_check_launch("mlstm_step");
 }

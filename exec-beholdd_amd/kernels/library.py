@@ -181,6 +181,7 @@ class KernelSizes:
             "bh_mlstm_gates": [p, p, f, p, ctypes.c_long, i, p, p, p, i, i, p],
             "bh_mlstm_scan": [p, i, i, i, i, i, p, p, ctypes.c_long, p, p, p, i, i, i, i, p],
             "bh_mlstm_finish": [p, p, p, i, i, i, p, f, p, i, i, i, i, p],
+            "bh_mlstm_step": [p, i, i, i, i, i, i, p, p, f, p, ctypes.c_long, p, p, f, p, i, i, i, i, i, p],
             "bh_softcap": [p, ctypes.c_long, f, p],
             "bh_rms_scale_add": [p, p, p, i, i, f, p],
             "bh_gelu_gate_table": [p, i, p, p, p, p, i, i, i, p, i, i, i, p],
@@ -1083,6 +1084,24 @@ class HipKernels(KernelSizes):
             self._ptr(read, "mlstm read", f32), self._ptr(beside, "mlstm beside", f32), self._ptr(proj, "mlstm gate"),
             _code(proj, "mlstm gate"), proj.shape[1], int(gate_off), self._ptr(weight, "mlstm norm weight", f32, True), float(eps),
             self._ptr(out, "mlstm out"), n_rows, n_heads, vdim, _block_rows(out), self._stream()))
+
+    def mlstm_step(self, proj, q_off, k_off, v_off, gate_off, pre, bias, cap, state, seq_slot, weight, eps, out, n_heads, dim, vdim):
+        """`mlstm_gates`, `mlstm_scan` and `mlstm_finish` in one launch for a step in which sequence b brings the one row b
+        (a decode step): the same arguments, the same numbers left in the slots' states, out [n, H vdim] in rows or blocks."""
+        n_rows = proj.shape[0]
+        width = n_heads * vdim
+        if seq_slot.shape != (n_rows,) or tuple(pre.shape) != (n_rows, 2 * n_heads) or tuple(out.shape) != (n_rows, width) \
+                or out.dtype != proj.dtype or state.dim() != 2 or state.shape[1] < self.mlstm_state_floats(n_heads, dim, vdim) \
+                or (bias is not None and tuple(bias.shape) != (2 * n_heads,)) or (weight is not None and tuple(weight.shape) != (width,)):
+            raise KernelError(f"mlstm_step: shapes proj {tuple(proj.shape)}, pre {tuple(pre.shape)}, state {tuple(state.shape)}, out "
+                              f"{tuple(out.shape)} do not fit {n_heads} heads of {dim} x {vdim} and a row a sequence")
+        f32, i32 = (torch.float32,), (torch.int32,)
+        self._check(self.lib.bh_mlstm_step(
+            self._ptr(proj, "mlstm proj"), _code(proj, "mlstm proj"), proj.shape[1], int(q_off), int(k_off), int(v_off), int(gate_off),
+            self._ptr(pre, "mlstm gates", f32), self._ptr(bias, "mlstm gate bias", f32, True), float(cap),
+            self._ptr(state, "mlstm state", f32), state.shape[1], self._ptr(seq_slot, "seq_slot", i32),
+            self._ptr(weight, "mlstm norm weight", f32, True), float(eps), self._ptr(out, "mlstm out"), n_rows, n_heads, dim, vdim,
+            _block_rows(out), self._stream()))
 
     def cast_concat(self, a, b, out):
         """out[r] = [a[r] | b[r]] in out's type; a, b f32 [n, D] (b may be None), out [n, 2 D] (or [n, D])."""

@@ -16,7 +16,8 @@ the state and both products of the recurrence are float32 in both engines.  Thre
 m of a sequence's rows in order and leaves exp(f + m' - m), exp(i - m) and m for every row; `mlstm_scan` walks the
 columns with those factors from the slot's state (prompts, portions and decode steps are one code path, so a
 position's result does not depend on the cut) and leaves S^T q and n . q; `mlstm_finish` divides, norms head by head
-and gates.  Every size and constant is a constructor parameter.
+and gates.  A step of one row a sequence (a decode step) does all three in one launch where the kernel set has it
+(`mlstm_step`).  Every size and constant is a constructor parameter.
 """
 
 from __future__ import annotations
@@ -79,13 +80,19 @@ class MatrixMemory:
         n, width = ctx.n_rows, self.n_heads * self.vdim
         proj = self.proj.forward(ctx, x)
         pre = self.gates.forward(ctx, x, out_dtype=torch.float32)
-        read = ctx.new_f32(n, width)                  # S^T q of every row and head
-        beside = ctx.new_f32(n, 4 * self.n_heads)     # the gates' two factors, m and n . q of every row and head
-        k.mlstm_gates(pre, self.gate_bias, self.gate_cap, cache.state, ctx.seq_start, ctx.seq_slot, beside, self.n_heads, self.dim, self.vdim)
-        k.mlstm_scan(proj, self.q_off, self.k_off, self.v_off, beside, cache.state, ctx.seq_start, ctx.seq_slot, read, self.n_heads,
-                     self.dim, self.vdim)
         gated = ctx.new_activations(n, width, reader=self.out.reader())
-        k.mlstm_finish(read, beside, proj, self.g_off, self.norm_weight, self.norm_eps, gated, self.n_heads, self.vdim)
+        one_launch = getattr(k, "mlstm_step", None)
+        if one_launch is not None and ctx.max_rows_per_seq == 1:      # a decode step: gates, recurrence and read-out in one launch
+            one_launch(proj, self.q_off, self.k_off, self.v_off, self.g_off, pre, self.gate_bias, self.gate_cap, cache.state, ctx.seq_slot,
+                       self.norm_weight, self.norm_eps, gated, self.n_heads, self.dim, self.vdim)
+        else:
+            read = ctx.new_f32(n, width)                  # S^T q of every row and head
+            beside = ctx.new_f32(n, 4 * self.n_heads)     # the gates' two factors, m and n . q of every row and head
+            k.mlstm_gates(pre, self.gate_bias, self.gate_cap, cache.state, ctx.seq_start, ctx.seq_slot, beside, self.n_heads, self.dim,
+                          self.vdim)
+            k.mlstm_scan(proj, self.q_off, self.k_off, self.v_off, beside, cache.state, ctx.seq_start, ctx.seq_slot, read, self.n_heads,
+                         self.dim, self.vdim)
+            k.mlstm_finish(read, beside, proj, self.g_off, self.norm_weight, self.norm_eps, gated, self.n_heads, self.vdim)
         self.out.forward(ctx, gated, out=hidden, accumulate=not fresh)
         return None
 

@@ -207,6 +207,45 @@ def test_matrix_memory(K, dtype, heads, dim, vdim, cap, lengths):
         assert rel(held[:, -1], kept[2]) < 1e-5
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads,dim,vdim,cap,seqs", [(3, 8, 20, 9.0, 4), (1, 16, 16, 1.0, 1), (4, 32, 40, 11.0, 9), (2, 80, 70, 15.0, 2),
+                                                     (5, 4, 15, 8.0, 3), (2, 128, 128, 12.0, 8), (1, 260, 16, 12.0, 2), (3, 12, 33, 6.0, 5)])
+def test_matrix_memory_decode_step_in_one_launch(K, dtype, heads, dim, vdim, cap, seqs):
+    """A step of one row a sequence through the one launch against the same step through the three kernels, from the states
+    that a ragged prompt left, into slots in another order than the batch's; three steps in a row."""
+    rng = np.random.default_rng(heads * vdim + dim + seqs)
+    key, value, eps = heads * dim, heads * vdim, 1e-5
+    lengths = [int(n) for n in rng.integers(1, 40, seqs)]
+    slots = list(rng.permutation(seqs + 1)[:seqs])
+    seq_start, seq_slot, _, _ = ragged(lengths, slots)
+    state = torch.zeros(seqs + 1, K.mlstm_state_floats(heads, dim, vdim) + 3, device="cuda:0")      # (a slot's row may be longer)
+    bias = dev(np.concatenate([rng.standard_normal(heads), rng.uniform(0.5, 4, heads)]).astype(np.float32))
+    norm_weight = dev((1 + 0.3 * rng.standard_normal(value)).astype(np.float32))
+
+    def three(proj, pre, state, seq_start):
+        n = proj.shape[0]
+        read, beside = torch.empty(n, value, device="cuda:0"), torch.empty(n, 4 * heads, device="cuda:0")
+        K.mlstm_gates(pre, bias, cap, state, seq_start, seq_slot, beside, heads, dim, vdim)
+        K.mlstm_scan(proj, 3, 3 + key, 3 + 2 * key, beside, state, seq_start, seq_slot, read, heads, dim, vdim)
+        out = torch.empty(n, value, dtype=dtype, device="cuda:0")
+        K.mlstm_finish(read, beside, proj, 3 + 2 * key + value, norm_weight, eps, out, heads, vdim)
+        return out
+    total = sum(lengths)
+    three(dev(rounded(rng.standard_normal((total, 3 + 2 * key + 2 * value)), dtype)[0]), dev((rng.standard_normal((total, 2 * heads)) * 3).astype(np.float32)),
+          state, seq_start)
+    other = state.clone()
+    one_each = dev(np.arange(seqs + 1, dtype=np.int32))
+    for _ in range(3):
+        proj = dev(rounded(rng.standard_normal((seqs, 3 + 2 * key + 2 * value)), dtype)[0])
+        pre = dev((rng.standard_normal((seqs, 2 * heads)) * 3).astype(np.float32))
+        want = three(proj, pre, state, one_each)
+        got = torch.empty(seqs, value, dtype=dtype, device="cuda:0")
+        K.mlstm_step(proj, 3, 3 + key, 3 + 2 * key, 3 + 2 * key + value, pre, bias, cap, other, seq_slot, norm_weight, eps, got, heads, dim, vdim)
+        assert rel(got, want.double().cpu().numpy()) < tol(dtype, f32=2e-5, bf16=8e-3)
+        assert rel(other, state.double().cpu().numpy()) < 1e-5
+    assert float(other[:, -3:].abs().max()) == 0
+
+
 # ---- the engine over every cut ------------------------------------------------------------------------------------
 
 @pytest.fixture(scope="module")
