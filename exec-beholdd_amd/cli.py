@@ -116,11 +116,11 @@ def _generate(args: list, out) -> int:
             raise UsageError(f"{path_flag}: {flags[path_flag]} exists and is never overwritten")
 
     from .config.base import read_config_json
-    from .registry import resolve_architecture
+    from .registry import configuration_of, resolve_architecture
 
     data, path = read_config_json(flags["--model"])
     entry = resolve_architecture(data, path)
-    config = entry.config_class.from_dict(data, path)
+    config = configuration_of(entry, data, path, flags["--model"])
     dtype = flags.get("--dtype", "bfloat16")
 
     if "--plan-only" in flags:

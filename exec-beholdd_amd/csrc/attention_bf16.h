@@ -51,4 +51,4 @@ __device__ inline u32x4_t keep_first(u32x4_t v, int n_valid) {
 void bh_attention_prefill_launch(const void* q, void* out, const void* k_pages, const void* v_pages,
                                  const int32_t* page_table, int table_stride, const int32_t* positions,
                                  const int32_t* seq_start, int n_seqs, int tiles, int H, int KVH, int hd,
-                                 float scale_log2, int window, int out_blocked, hipStream_t stream);
+                                 float scale_log2, int window, int out_blocked, const float* sinks, hipStream_t stream);

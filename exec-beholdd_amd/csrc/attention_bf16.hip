@@ -144,7 +144,7 @@ __global__ __launch_bounds__(256, (LEAN ? 2 : 1)) void attention_mfma_kernel(
     float* __restrict__ part_ml, const uint16_t* __restrict__ k_pages, const uint16_t* __restrict__ v_pages,
     const int32_t* __restrict__ page_table, int table_stride, const int32_t* __restrict__ positions,
     const int32_t* __restrict__ seq_start, int H, int KVH, float scale_log2, int window, int n_splits,
-    int pages_per_split, int tile_groups, FusedQkv fused, int out_block_rows) {
+    int pages_per_split, int tile_groups, FusedQkv fused, int out_block_rows, const float* __restrict__ sinks) {
   constexpr int HD = 32 * NS;
   __shared__ float sm_m[4][16];
   __shared__ float sm_l[4][16];
@@ -401,6 +401,8 @@ __global__ __launch_bounds__(256, (LEAN ? 2 : 1)) void attention_mfma_kernel(
       }
       const size_t column = (size_t)(row0 + cc / G) * H + kvh * G + cc % G;
       if (n_splits == 1) {   // out_block_rows: the output [rows][H * HD] lies in blocks of that many rows (bh_rows_index)
+        // a sink: one more term exp(sinks[head]) in the softmax's sum (`top` is in powers of two)
+        if (sinks) sum += exp2f(sinks[kvh * G + cc % G] * 1.4426950408889634f - safe_top);
         out[bh_rows_index(out_block_rows, row0 + cc / G, (kvh * G + cc % G) * HD + d, H * HD)] = f32_to_bf16_bits(value / sum);
       } else {
         part_o[(column * n_splits + split) * HD + d] = value;
@@ -419,7 +421,8 @@ __global__ __launch_bounds__(256, (LEAN ? 2 : 1)) void attention_mfma_kernel(
 // no more); the sums run over the splits in their order either way.
 template <int WIDTH>
 __global__ void attention_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                         uint16_t* __restrict__ out, int n_splits, int HD, int H, int out_block_rows) {
+                                         uint16_t* __restrict__ out, int n_splits, int HD, int H, int out_block_rows,
+                                         const float* __restrict__ sinks) {
   const size_t column = blockIdx.x;
   const float* ml = part_ml + column * n_splits * 2;
   const int lane = threadIdx.x % BH_WAVE;
@@ -436,6 +439,7 @@ __global__ void attention_combine_kernel(const float* __restrict__ part_o, const
   for (int s = lane; s < n_splits; s += BH_WAVE) sum += ml[2 * s + 1] * exp2f(ml[2 * s] - top);
 #pragma unroll
   for (int off = BH_WAVE / 2; off > 0; off >>= 1) sum += __shfl_xor(sum, off, BH_WAVE);
+  if (sinks) sum += exp2f(sinks[column % H] * 1.4426950408889634f - top);      // the sink's term, once for the whole row
   const float inv = 1.0f / sum;
   for (int d = threadIdx.x; d < HD; d += blockDim.x) {
     float value = 0.f;
@@ -510,7 +514,7 @@ static int attention_bf16_run(const void* q, void* out, void* part_o, void* part
                               const int32_t* positions, const int32_t* seq_start, int n_seqs, int n_rows,
                               int max_rows_per_seq, int H, int KVH, int hd, float scale, int window,
                               int max_position, int n_splits, const FusedQkv& fused, int out_blocked,
-                              hipStream_t stream) {
+                              const float* sinks, hipStream_t stream) {
   BH_REQUIRE(n_seqs > 0 && n_rows > 0 && max_rows_per_seq > 0, "attention_bf16: empty batch");
   BH_REQUIRE(H > 0 && KVH > 0 && H % KVH == 0, "attention_bf16: %d query heads do not group evenly into %d kv heads", H, KVH);
   BH_REQUIRE(hd % 32 == 0 && hd >= 32 && hd <= 256, "attention_bf16: head size %d is not a multiple of 32 up to 256", hd);
@@ -528,7 +532,7 @@ static int attention_bf16_run(const void* q, void* out, void* part_o, void* part
   if (!is_fused && n_splits == 1 && (long)tiles * KVH * n_seqs >= PREFILL_FROM_TILES) {   // many columns: the prefill kernel
     BH_REQUIRE(out_blocked == 0 || out_blocked == 16, "attention_bf16: a step of many columns writes rows or blocks of 16 rows, not of %d", out_blocked);
     bh_attention_prefill_launch(q, out, k_pages, v_pages, page_table, table_stride, positions, seq_start, n_seqs,
-                                tiles, H, KVH, hd, scale_log2, window, out_blocked == 16, stream);
+                                tiles, H, KVH, hd, scale_log2, window, out_blocked == 16, sinks, stream);
     return bh_check_launch("attention_prefill_bf16");
   }
   BH_REQUIRE(out_blocked == 0 || ((out_blocked == 8 || out_blocked == 16) && (H * hd) % 32 == 0),
@@ -540,7 +544,7 @@ static int attention_bf16_run(const void* q, void* out, void* part_o, void* part
   attention_mfma_kernel<NS, STREAM, FUSED, ##__VA_ARGS__><<<grid, block, 0, stream>>>(                          \
       (const uint16_t*)q, (uint16_t*)out, (float*)part_o, (float*)part_ml, (const uint16_t*)k_pages,            \
       (const uint16_t*)v_pages, page_table, table_stride, positions, seq_start, H, KVH, scale_log2, window,     \
-      n_splits, per, tile_groups, fused, out_blocked)
+      n_splits, per, tile_groups, fused, out_blocked, sinks)
 #define BH_ATT(NS)                                      \
   do {                                                  \
     if (is_fused && lean && NS <= 4) BH_ATT_ONE(NS, true, true, (NS <= 4));   \
@@ -565,10 +569,10 @@ static int attention_bf16_run(const void* q, void* out, void* part_o, void* part
     const dim3 columns(n_rows * H), threads(hd >= 128 ? 128 : 64);
     if (n_splits <= 4)
       attention_combine_kernel<4><<<columns, threads, 0, stream>>>((const float*)part_o, (const float*)part_ml, (uint16_t*)out,
-                                                                   n_splits, hd, H, out_blocked);
+                                                                   n_splits, hd, H, out_blocked, sinks);
     else
       attention_combine_kernel<8><<<columns, threads, 0, stream>>>((const float*)part_o, (const float*)part_ml, (uint16_t*)out,
-                                                                   n_splits, hd, H, out_blocked);
+                                                                   n_splits, hd, H, out_blocked, sinks);
     return bh_check_launch("attention_combine");
   }
   return 0;
@@ -578,11 +582,11 @@ extern "C" int bh_attention_bf16(const void* q, void* out, void* part_o, void* p
                                  const void* v_pages, const int32_t* page_table, int table_stride,
                                  const int32_t* positions, const int32_t* seq_start, int n_seqs, int n_rows,
                                  int max_rows_per_seq, int H, int KVH, int hd, float scale, int window,
-                                 int max_position, int n_splits, int out_blocked, hipStream_t stream) {
+                                 int max_position, int n_splits, int out_blocked, const float* sinks, hipStream_t stream) {
   const FusedQkv none = {nullptr, nullptr, nullptr, 0, 0.f, nullptr, nullptr, 0, nullptr, nullptr};
   return attention_bf16_run(q, out, part_o, part_ml, k_pages, v_pages, page_table, table_stride, positions,
                             seq_start, n_seqs, n_rows, max_rows_per_seq, H, KVH, hd, scale, window, max_position,
-                            n_splits, none, out_blocked, stream);
+                            n_splits, none, out_blocked, sinks, stream);
 }
 
 // A decode step (one row per sequence) straight from the fused projection rows [q heads | k heads | v heads]:
@@ -609,5 +613,5 @@ extern "C" int bh_attention_decode_fused(const void* qkv, void* out, void* part_
                           write_kv, (uint16_t*)k_pages, (uint16_t*)v_pages};
   return attention_bf16_run(nullptr, out, part_o, part_ml, k_pages, v_pages, page_table, table_stride, positions,
                             seq_start, n_seqs, n_seqs, 1, H, KVH, hd, scale, window, max_position, n_splits, fused,
-                            out_block_rows, stream);
+                            out_block_rows, nullptr, stream);
 }

@@ -53,7 +53,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NS <= 4 ? 2
     const uint16_t* __restrict__ q, uint16_t* __restrict__ out, const uint16_t* __restrict__ k_pages,
     const uint16_t* __restrict__ v_pages, const int32_t* __restrict__ page_table, int table_stride,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ seq_start, int H, int KVH,
-    float scale_log2, int window, int tile_groups, int n_seqs, int out_blocked) {
+    float scale_log2, int window, int tile_groups, int n_seqs, int out_blocked, const float* __restrict__ sinks) {
   constexpr int HD = 32 * NS;
   constexpr int PIECES = BH_PAGE * HD / 8;        // 16-byte pieces of one head's keys (or values) in a page
   constexpr int STAGE = 2 * PIECES / 256;         // pieces of a page (keys, then values) one thread copies
@@ -320,7 +320,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NS <= 4 ? 2
   for (int ct = 0; ct < CTW; ++ct) {
     const int cc = (wave_tile0 + ct) * 16 + j;
     if (cc >= n_cols) continue;
-    const float inv = 1.0f / run_sum[ct][0];
+    // a sink: one more term exp(sinks[head]) in the softmax's sum, taken against the exponentials' reference
+    const float sunk = sinks ? __builtin_amdgcn_exp2f((sinks[kvh * G + cc % G] * 1.4426950408889634f) - run_max[ct] * scale_log2) : 0.f;
+    const float inv = 1.0f / (run_sum[ct][0] + sunk);
     const int out_row = row0 + cc / G, out_column = (kvh * G + cc % G) * HD + 4 * g;
 #pragma unroll
     for (int dt = 0; dt < 2 * NS; ++dt) {
@@ -339,13 +341,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(NS <= 4 ? 2
 void bh_attention_prefill_launch(const void* q, void* out, const void* k_pages, const void* v_pages,
                                  const int32_t* page_table, int table_stride, const int32_t* positions,
                                  const int32_t* seq_start, int n_seqs, int tiles, int H, int KVH, int hd,
-                                 float scale_log2, int window, int out_blocked, hipStream_t stream) {
+                                 float scale_log2, int window, int out_blocked, const float* sinks, hipStream_t stream) {
 #define BH_PREFILL(NS, CTW)                                                                                  \
   do {                                                                                                       \
     const int tile_groups = (tiles + 4 * CTW - 1) / (4 * CTW);                                               \
     attention_prefill_kernel<NS, CTW><<<dim3(tile_groups * KVH * n_seqs), dim3(256), 0, stream>>>(           \
         (const uint16_t*)q, (uint16_t*)out, (const uint16_t*)k_pages, (const uint16_t*)v_pages, page_table,  \
-        table_stride, positions, seq_start, H, KVH, scale_log2, window, tile_groups, n_seqs, out_blocked);   \
+        table_stride, positions, seq_start, H, KVH, scale_log2, window, tile_groups, n_seqs, out_blocked, sinks); \
   } while (0)
   // Two column tiles per wave while the accumulators leave room for two workgroups per compute unit; one
   // where that gives fewer than two workgroups per compute unit (a page costs a workgroup nearly the same

@@ -4,14 +4,17 @@
 //   experts_gate_up    per (row, chosen expert): inner = act(Wg_e h, Wu_e h)             (weights read per pair: the
 //   experts_down       per row: h_res += sum_j weight_j * Wd_ej inner_j, j in order       form for steps of few rows)
 //   clamped_glu        act over a stacked [gate | up] matrix (the shared expert, and experts run as products of rows)
-//   act(g, u) = g' * sigmoid(alpha g') * (u' + 1),  g' = min(g, limit),  u' = clamp(u, -limit, limit)
+//   act(g, u) = g' * sigmoid(alpha g') * (u' + shift),  g' = min(g, limit),  u' = clamp(u, -limit, limit)
+//               (an infinite limit, alpha 1 and shift 0 give silu(g) * u)
+// A router may score by the sigmoid of every chosen logit instead (`scoring` 1), and a pair's weight may multiply the
+// expert's input instead of its output: W (w h) = w (W h), so the gate and up sums are multiplied ahead of the activation.
 // Router logits, the softmax and all sums are float32.
 #include "common.h"
 
-__device__ inline float clamped_glu(float g, float u, float limit, float alpha) {
+__device__ inline float clamped_glu(float g, float u, float limit, float alpha, float shift) {
   g = fminf(g, limit);
   u = fminf(fmaxf(u, -limit), limit);
-  return g / (1.0f + expf(-alpha * g)) * (u + 1.0f);
+  return g / (1.0f + expf(-alpha * g)) * (u + shift);
 }
 
 #define ROUTE_MAX_TOP 32
@@ -21,7 +24,7 @@ __device__ inline float clamped_glu(float g, float u, float limit, float alpha) 
 // without those already taken (ties go to the lower index).
 __global__ __launch_bounds__(256) void route_top_k_kernel(const float* __restrict__ logits, const float* __restrict__ bias,
                                                          int32_t* __restrict__ chosen, float* __restrict__ weights, int n_rows,
-                                                         int E, int top) {
+                                                         int E, int top, int scoring) {
   const int lane = threadIdx.x & (BH_WAVE - 1), row = blockIdx.x * (blockDim.x / BH_WAVE) + threadIdx.x / BH_WAVE;
   if (row >= n_rows) return;
   const float* z = logits + (size_t)row * E;
@@ -56,7 +59,7 @@ __global__ __launch_bounds__(256) void route_top_k_kernel(const float* __restric
     }
     if ((best_e & (BH_WAVE - 1)) == lane) taken |= 1u << (best_e / BH_WAVE);
     if (j == 0) largest = best;
-    const float p = expf(best - largest);
+    const float p = scoring ? 1.0f / (1.0f + expf(-best)) : expf(best - largest);
     sum += p;
     if (lane == j) {
       mine = p;
@@ -65,15 +68,15 @@ __global__ __launch_bounds__(256) void route_top_k_kernel(const float* __restric
   }
   if (lane < top) {
     chosen[(size_t)row * top + lane] = mine_index;
-    weights[(size_t)row * top + lane] = mine / sum;
+    weights[(size_t)row * top + lane] = scoring ? mine : mine / sum;
   }
 }
 
 extern "C" int bh_route_top_k(const float* logits, const float* bias, int32_t* chosen, float* weights, int n_rows, int E, int top,
-                              hipStream_t stream) {
+                              int scoring, hipStream_t stream) {
   BH_REQUIRE(n_rows > 0 && E > 0 && E <= BH_WAVE * ROUTE_PER_LANE, "route_top_k: 1 to %d experts, got %d", BH_WAVE * ROUTE_PER_LANE, E);
   BH_REQUIRE(top >= 1 && top <= E && top <= ROUTE_MAX_TOP, "route_top_k: 1 to min(%d, %d) experts a row, got %d", E, ROUTE_MAX_TOP, top);
-  route_top_k_kernel<<<(n_rows + 3) / 4, 256, 0, stream>>>(logits, bias, chosen, weights, n_rows, E, top);
+  route_top_k_kernel<<<(n_rows + 3) / 4, 256, 0, stream>>>(logits, bias, chosen, weights, n_rows, E, top, scoring);
   return bh_check_launch("route_top_k");
 }
 
@@ -101,7 +104,8 @@ __device__ inline float wave_dot(const T* __restrict__ w, const float* __restric
 template <typename T>
 __global__ __launch_bounds__(256) void experts_gate_up_kernel(const T* __restrict__ h, const int32_t* __restrict__ chosen,
                                                               const T* __restrict__ w_gu, T* __restrict__ inner, int top, int K, int ff,
-                                                              float limit, float alpha) {
+                                                              float limit, float alpha, float shift,
+                                                              const float* __restrict__ in_weights) {
   extern __shared__ float xs[];
   const int pair = blockIdx.x, row = pair / top, e = chosen[pair];
   for (int k = threadIdx.x; k < K; k += blockDim.x) xs[k] = to_f32(h[(size_t)row * K + k]);
@@ -113,12 +117,13 @@ __global__ __launch_bounds__(256) void experts_gate_up_kernel(const T* __restric
     if (o >= ff) break;
     const float g = wave_dot(base + (size_t)o * K, xs, K, lane);
     const float u = wave_dot(base + (size_t)(ff + o) * K, xs, K, lane);
-    if (lane == 0) inner[(size_t)pair * ff + o] = from_f32<T>(clamped_glu(g, u, limit, alpha));
+    const float wgt = in_weights ? in_weights[pair] : 1.0f;
+    if (lane == 0) inner[(size_t)pair * ff + o] = from_f32<T>(clamped_glu(g * wgt, u * wgt, limit, alpha, shift));
   }
 }
 
 extern "C" int bh_experts_gate_up(const void* h, int dtype, const int32_t* chosen, const void* w_gu, void* inner, int n_rows, int top,
-                                  int K, int ff, float limit, float alpha, hipStream_t stream) {
+                                  int K, int ff, float limit, float alpha, float shift, const float* in_weights, hipStream_t stream) {
   BH_REQUIRE(n_rows > 0 && top > 0 && K > 0 && ff > 0, "experts_gate_up: sizes must be positive");
   BH_REQUIRE((size_t)K * sizeof(float) <= 64 * 1024, "experts_gate_up: rows of up to 16384 inputs, got %d", K);
   dim3 grid(n_rows * top, (ff + EX_OUTS - 1) / EX_OUTS);
@@ -127,10 +132,10 @@ extern "C" int bh_experts_gate_up(const void* h, int dtype, const int32_t* chose
   if (dtype == BH_BF16) bh_allow_lds<experts_gate_up_kernel<bf16_t>>(lds);
   if (dtype == BH_F32)
     experts_gate_up_kernel<float><<<grid, 64 * EX_WAVES, lds, stream>>>((const float*)h, chosen, (const float*)w_gu, (float*)inner, top, K, ff,
-                                                                       limit, alpha);
+                                                                       limit, alpha, shift, in_weights);
   else if (dtype == BH_BF16)
     experts_gate_up_kernel<bf16_t><<<grid, 64 * EX_WAVES, lds, stream>>>((const bf16_t*)h, chosen, (const bf16_t*)w_gu, (bf16_t*)inner, top, K,
-                                                                        ff, limit, alpha);
+                                                                        ff, limit, alpha, shift, in_weights);
   else
     return bh_fail("experts_gate_up: unknown dtype %d", dtype);
   return bh_check_launch("experts_gate_up");
@@ -152,7 +157,7 @@ __global__ __launch_bounds__(256) void experts_down_kernel(const T* __restrict__
     float total = 0.f;
     for (int j = 0; j < top; ++j) {
       const int e = chosen[(size_t)row * top + j];
-      total = fmaf(weights[(size_t)row * top + j], wave_dot(w_d + ((size_t)e * D + o) * ff, xs + (size_t)j * ff, ff, lane), total);
+      total = fmaf(weights ? weights[(size_t)row * top + j] : 1.0f, wave_dot(w_d + ((size_t)e * D + o) * ff, xs + (size_t)j * ff, ff, lane), total);
     }
     if (lane == 0) hidden[(size_t)row * D + o] += total;
   }
@@ -178,26 +183,26 @@ extern "C" int bh_experts_down(const void* inner, int dtype, const int32_t* chos
 
 template <typename T>
 __global__ __launch_bounds__(256) void clamped_glu_kernel(const T* __restrict__ gu, T* __restrict__ out, int n_rows, int ff, float limit,
-                                                          float alpha, int out_block_rows) {
+                                                          float alpha, int out_block_rows, float shift) {
   const size_t n = (size_t)n_rows * ff;
   for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (size_t)gridDim.x * blockDim.x) {
     const int r = (int)(e / ff), i = (int)(e % ff);
     const float g = to_f32(gu[(size_t)r * 2 * ff + i]), u = to_f32(gu[(size_t)r * 2 * ff + ff + i]);
-    out[bh_rows_index(out_block_rows, r, i, ff)] = from_f32<T>(clamped_glu(g, u, limit, alpha));
+    out[bh_rows_index(out_block_rows, r, i, ff)] = from_f32<T>(clamped_glu(g, u, limit, alpha, shift));
   }
 }
 
 extern "C" int bh_clamped_glu(const void* gu, int dtype, void* out, int n_rows, int ff, float limit, float alpha, int out_block_rows,
-                              hipStream_t stream) {
+                              float shift, hipStream_t stream) {
   BH_REQUIRE(n_rows > 0 && ff > 0, "clamped_glu: sizes must be positive");
   BH_REQUIRE(out_block_rows == 0 || ((out_block_rows == 8 || out_block_rows == 16) && ff % 32 == 0 && dtype == BH_BF16),
              "clamped_glu: rows in blocks of %d of width %d are not written", out_block_rows, ff);
   const size_t n = (size_t)n_rows * ff;
   const int blocks = (int)((n + 255) / 256 < 8192 ? (n + 255) / 256 : 8192);
   if (dtype == BH_F32)
-    clamped_glu_kernel<float><<<blocks, 256, 0, stream>>>((const float*)gu, (float*)out, n_rows, ff, limit, alpha, out_block_rows);
+    clamped_glu_kernel<float><<<blocks, 256, 0, stream>>>((const float*)gu, (float*)out, n_rows, ff, limit, alpha, out_block_rows, shift);
   else if (dtype == BH_BF16)
-    clamped_glu_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, n_rows, ff, limit, alpha, out_block_rows);
+    clamped_glu_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, n_rows, ff, limit, alpha, out_block_rows, shift);
   else
     return bh_fail("clamped_glu: unknown dtype %d", dtype);
   return bh_check_launch("clamped_glu");
@@ -270,7 +275,8 @@ __device__ inline void load8<bf16_t>(const bf16_t* __restrict__ p, float (&v)[8]
 template <typename T, bool GATED, int U>
 __global__ __launch_bounds__(256) void experts_rows_kernel(const T* __restrict__ in, int in_div, const int32_t* __restrict__ list, int capacity,
                                                            const int32_t* __restrict__ counts, const T* __restrict__ w, void* __restrict__ out_raw,
-                                                           int K, int N, float limit, float alpha) {
+                                                           int K, int N, float limit, float alpha, float shift,
+                                                           const float* __restrict__ in_weights) {
   const int e = blockIdx.x, count = counts[e];
   if (count == 0) return;
   const int lane = threadIdx.x & (BH_WAVE - 1), wave = threadIdx.x / BH_WAVE;
@@ -324,7 +330,8 @@ __global__ __launch_bounds__(256) void experts_rows_kernel(const T* __restrict__
           const float b = GATED ? wave_sum(acc_b[u][j]) : 0.f;
           if (lane == 0 && o0 + u < N) {
             const size_t at = (size_t)mine[p0 + j] * N + o0 + u;
-            if (GATED) reinterpret_cast<T*>(out_raw)[at] = from_f32<T>(clamped_glu(a, b, limit, alpha));
+            const float wgt = (GATED && in_weights) ? in_weights[mine[p0 + j]] : 1.0f;
+            if (GATED) reinterpret_cast<T*>(out_raw)[at] = from_f32<T>(clamped_glu(a * wgt, b * wgt, limit, alpha, shift));
             else reinterpret_cast<float*>(out_raw)[at] = a;
           }
         }
@@ -334,11 +341,12 @@ __global__ __launch_bounds__(256) void experts_rows_kernel(const T* __restrict__
 }
 
 extern "C" int bh_experts_rows(const void* in, int dtype, int in_div, const int32_t* list, int capacity, const int32_t* counts, const void* w,
-                               void* out, int E, int K, int N, int gated, float limit, float alpha, hipStream_t stream) {
+                               void* out, int E, int K, int N, int gated, float limit, float alpha, float shift, const float* in_weights,
+                               hipStream_t stream) {
   BH_REQUIRE(E > 0 && K > 0 && N > 0 && in_div > 0 && capacity > 0, "experts_rows: sizes must be positive");
   BH_REQUIRE(K % 8 == 0, "experts_rows: rows of a multiple of 8 inputs, got %d", K);
   dim3 grid(E, (N + ER_OUTS - 1) / ER_OUTS);
-#define BH_ER(T, G, U) experts_rows_kernel<T, G, U><<<grid, 256, 0, stream>>>((const T*)in, in_div, list, capacity, counts, (const T*)w, out, K, N, limit, alpha)
+#define BH_ER(T, G, U) experts_rows_kernel<T, G, U><<<grid, 256, 0, stream>>>((const T*)in, in_div, list, capacity, counts, (const T*)w, out, K, N, limit, alpha, shift, in_weights)
   if (dtype == BH_F32) {
     if (gated) BH_ER(float, true, 2);
     else BH_ER(float, false, 4);
@@ -356,25 +364,32 @@ extern "C" int bh_experts_rows(const void* in, int dtype, int in_div, const int3
 template <typename T>
 __global__ __launch_bounds__(256) void experts_gather_kernel(const T* __restrict__ x, int top, const int32_t* __restrict__ list, int capacity,
                                                              const int32_t* __restrict__ counts, const int32_t* __restrict__ offsets,
-                                                             T* __restrict__ sorted, int32_t* __restrict__ place, int K) {
+                                                             T* __restrict__ sorted, int32_t* __restrict__ place, int K,
+                                                             const float* __restrict__ in_weights) {
   const int e = blockIdx.x, count = counts[e], first = offsets[e];
   for (int i = blockIdx.y; i < count; i += gridDim.y) {
     const int pair = list[(size_t)e * capacity + i];
     const T* from = x + (size_t)(pair / top) * K;
     T* to = sorted + (size_t)(first + i) * K;
-    for (int k = threadIdx.x; k < K; k += blockDim.x) to[k] = from[k];
+    if (in_weights) {      // the pair's weight on the expert's input
+      const float wgt = in_weights[pair];
+      for (int k = threadIdx.x; k < K; k += blockDim.x) to[k] = from_f32<T>(to_f32(from[k]) * wgt);
+    } else {
+      for (int k = threadIdx.x; k < K; k += blockDim.x) to[k] = from[k];
+    }
     if (threadIdx.x == 0) place[pair] = first + i;
   }
 }
 
 extern "C" int bh_experts_gather(const void* x, int dtype, int top, const int32_t* list, int capacity, const int32_t* counts,
-                                 const int32_t* offsets, void* sorted, int32_t* place, int E, int K, int n_rows, hipStream_t stream) {
+                                 const int32_t* offsets, void* sorted, int32_t* place, int E, int K, int n_rows, const float* in_weights,
+                                 hipStream_t stream) {
   BH_REQUIRE(E > 0 && K > 0 && top > 0 && n_rows > 0, "experts_gather: sizes must be positive");
   dim3 grid(E, n_rows < 256 ? n_rows : 256);
   if (dtype == BH_F32)
-    experts_gather_kernel<float><<<grid, 256, 0, stream>>>((const float*)x, top, list, capacity, counts, offsets, (float*)sorted, place, K);
+    experts_gather_kernel<float><<<grid, 256, 0, stream>>>((const float*)x, top, list, capacity, counts, offsets, (float*)sorted, place, K, in_weights);
   else if (dtype == BH_BF16)
-    experts_gather_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)x, top, list, capacity, counts, offsets, (bf16_t*)sorted, place, K);
+    experts_gather_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)x, top, list, capacity, counts, offsets, (bf16_t*)sorted, place, K, in_weights);
   else
     return bh_fail("experts_gather: unknown dtype %d", dtype);
   return bh_check_launch("experts_gather");
@@ -388,7 +403,7 @@ __global__ __launch_bounds__(256) void experts_combine_kernel(const float* __res
   float total = 0.f;
   for (int j = 0; j < top; ++j) {
     const int pair = row * top + j;
-    total = fmaf(weights[pair], y[(size_t)(place ? place[pair] : pair) * D + d], total);
+    total = fmaf(weights ? weights[pair] : 1.0f, y[(size_t)(place ? place[pair] : pair) * D + d], total);
   }
   hidden[(size_t)row * D + d] += total;
 }

@@ -26,16 +26,16 @@ __device__ inline em_bf16x8_t em_operand(const uint16_t* p) {
   return u.v;
 }
 
-__device__ inline float em_act(float g, float u, float limit, float alpha) {
+__device__ inline float em_act(float g, float u, float limit, float alpha, float shift) {
   g = fminf(g, limit);
   u = fminf(fmaxf(u, -limit), limit);
-  return g / (1.0f + expf(-alpha * g)) * (u + 1.0f);
+  return g / (1.0f + expf(-alpha * g)) * (u + shift);
 }
 
 template <bool GATED>
 __global__ __launch_bounds__(256) void experts_products_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ w,
                                                                const int32_t* __restrict__ tiles, void* __restrict__ out_raw, int K,
-                                                               int N, float limit, float alpha) {
+                                                               int N, float limit, float alpha, float shift) {
   __shared__ __align__(16) uint16_t lds_a[EM_TILE * EM_PITCH];
   __shared__ __align__(16) uint16_t lds_b[EM_TILE * EM_PITCH];
   const int expert = tiles[3 * blockIdx.x], first = tiles[3 * blockIdx.x + 1], rows = tiles[3 * blockIdx.x + 2];
@@ -107,7 +107,7 @@ __global__ __launch_bounds__(256) void experts_products_kernel(const uint16_t* _
       for (int y = 0; y < 2; ++y) {
         const int n = n0 + y * 32 + (lane & 31);
         if (n < N)
-          reinterpret_cast<bf16_t*>(out_raw)[(size_t)(first + row) * N + n] = from_f32<bf16_t>(em_act(acc[y][i], acc[y + 2][i], limit, alpha));
+          reinterpret_cast<bf16_t*>(out_raw)[(size_t)(first + row) * N + n] = from_f32<bf16_t>(em_act(acc[y][i], acc[y + 2][i], limit, alpha, shift));
       }
     } else {
 #pragma unroll
@@ -125,14 +125,14 @@ extern "C" int bh_experts_products_takes(int K, int N) { return K > 0 && N > 0 &
 // a bfloat16 [rows][K]; w bfloat16 [E][gated ? 2 N : N][K]; tiles int32 [n_tiles][3] = {expert, first row, rows (1..128)} on the
 // device; out bfloat16 [rows][N] (gated) or float32 [rows][N].
 extern "C" int bh_experts_products(const void* a, const void* w, const int32_t* tiles, int n_tiles, void* out, int K, int N, int gated,
-                                   float limit, float alpha, hipStream_t stream) {
+                                   float limit, float alpha, float shift, hipStream_t stream) {
   BH_REQUIRE(n_tiles > 0 && bh_experts_products_takes(K, N), "experts_products: K must be a multiple of %d, got %d", EM_K, K);
   const int outs = gated ? EM_TILE / 2 : EM_TILE;
   dim3 grid(n_tiles, (N + outs - 1) / outs);
   BH_REQUIRE(grid.y <= 65535, "experts_products: too many outputs");
   if (gated)
-    experts_products_kernel<true><<<grid, 256, 0, stream>>>((const uint16_t*)a, (const uint16_t*)w, tiles, out, K, N, limit, alpha);
+    experts_products_kernel<true><<<grid, 256, 0, stream>>>((const uint16_t*)a, (const uint16_t*)w, tiles, out, K, N, limit, alpha, shift);
   else
-    experts_products_kernel<false><<<grid, 256, 0, stream>>>((const uint16_t*)a, (const uint16_t*)w, tiles, out, K, N, limit, alpha);
+    experts_products_kernel<false><<<grid, 256, 0, stream>>>((const uint16_t*)a, (const uint16_t*)w, tiles, out, K, N, limit, alpha, shift);
   return bh_check_launch("experts_products");
 }

@@ -740,7 +740,8 @@ template <typename T, int THREADS>
 __global__ __launch_bounds__(THREADS) void attention_generic_kernel(
     const T* __restrict__ q, T* __restrict__ out, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
     const int32_t* __restrict__ page_table, int table_stride, const int32_t* __restrict__ row_seq,
-    const int32_t* __restrict__ positions, int H, int KVH, int hd, float scale, int window, int kv_order) {
+    const int32_t* __restrict__ positions, int H, int KVH, int hd, float scale, int window, int kv_order,
+    const float* __restrict__ sinks) {
   extern __shared__ float smem[];
   float* qs = smem;                    // [hd]
   float* probs = qs + hd;              // [THREADS]
@@ -798,14 +799,16 @@ __global__ __launch_bounds__(THREADS) void attention_generic_kernel(
   if (tid < hd) {
     float total = 0.f;
     for (int g = 0; g < n_groups; ++g) total += partial[g * hd + tid];
-    out[((size_t)row * H + head) * hd + tid] = from_f32<T>(total / run_sum);
+    // a sink: one more term exp(sinks[head]) in the softmax's sum, with no key and no value
+    const float all = sinks ? run_sum + expf(sinks[head] - run_max) : run_sum;
+    out[((size_t)row * H + head) * hd + tid] = from_f32<T>(total / all);
   }
 }
 
 extern "C" int bh_attention_generic(const void* q, void* out, int dtype, const void* k_pages,
                                     const void* v_pages, const int32_t* page_table, int table_stride,
                                     const int32_t* row_seq, const int32_t* positions, int n_rows, int H,
-                                    int KVH, int hd, float scale, int window, int kv_order,
+                                    int KVH, int hd, float scale, int window, int kv_order, const float* sinks,
                                     hipStream_t stream) {
   BH_REQUIRE(n_rows > 0 && H > 0 && KVH > 0 && hd > 0, "attention: sizes must be positive");
   BH_REQUIRE(H % KVH == 0, "attention: %d query heads do not group evenly into %d kv heads", H, KVH);
@@ -819,7 +822,7 @@ extern "C" int bh_attention_generic(const void* q, void* out, int dtype, const v
 #define BH_AG(T, THREADS)                                                                                             \
   attention_generic_kernel<T, THREADS><<<grid, block, smem, stream>>>((const T*)q, (T*)out, (const T*)k_pages, (const T*)v_pages, \
                                                                       page_table, table_stride, row_seq, positions, H, KVH, hd,  \
-                                                                      scale, window, kv_order)
+                                                                      scale, window, kv_order, sinks)
 #define BH_AG_SIZES(T)                        \
   do {                                        \
     if (threads == AG_THREADS) BH_AG(T, AG_THREADS); \

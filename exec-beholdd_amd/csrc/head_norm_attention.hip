@@ -21,7 +21,7 @@ __global__ __launch_bounds__(HN_WAVES * BH_WAVE) void head_norm_rope_write_kerne
     const float* __restrict__ wk, float eps, const float* __restrict__ freq, int turned, const int32_t* __restrict__ positions,
     const int32_t* __restrict__ row_seq, T* __restrict__ q_out, T* __restrict__ k_pages, T* __restrict__ v_pages,
     const int32_t* __restrict__ page_table, int table_stride, int H, int G, int dim, int vdim, int pad, int kv_order, int write,
-    int per_group) {
+    int per_group, int neighbours, float magnitude) {
   extern __shared__ float lds[];      // the cosines and sines of the row's turned pairs, then a head of `dim` floats a wave
   const int row = blockIdx.x, wave = threadIdx.x / BH_WAVE, lane = threadIdx.x % BH_WAVE;
   const int half = turned / 2;
@@ -31,8 +31,8 @@ __global__ __launch_bounds__(HN_WAVES * BH_WAVE) void head_norm_rope_write_kerne
   const int pos = positions[row];
   for (int i = threadIdx.x; i < half; i += blockDim.x) {
     const float angle = (float)pos * freq[i];
-    cosines[i] = cosf(angle);
-    sines[i] = sinf(angle);
+    cosines[i] = cosf(angle) * magnitude;
+    sines[i] = sinf(angle) * magnitude;
   }
   __syncthreads();
   const T* x = proj + (size_t)row * row_stride + first;
@@ -72,10 +72,13 @@ __global__ __launch_bounds__(HN_WAVES * BH_WAVE) void head_norm_rope_write_kerne
       if (i < dim) {
         y = mine[i] * inv * (w ? w[i] : 1.f);
         if (i < turned) {
-          const int pair = i < half ? i : i - half, mate = i < half ? i + half : i - half;
+          // the pair's mate: i + half and i - half, or the neighbour (2 pair, 2 pair + 1)
+          const int pair = neighbours ? i / 2 : (i < half ? i : i - half);
+          const bool is_first = neighbours ? (i % 2 == 0) : (i < half);
+          const int mate = neighbours ? (i ^ 1) : (i < half ? i + half : i - half);
           const float other = mine[mate] * inv * (w ? w[mate] : 1.f);
           const float c = cosines[pair], s = sines[pair];
-          y = i < half ? y * c - other * s : y * c + other * s;
+          y = is_first ? y * c - other * s : y * c + other * s;
         }
       }
       if (is_key) keys[bh_key_index(kv_order, token, i, pad)] = from_f32<T>(y);
@@ -87,12 +90,13 @@ __global__ __launch_bounds__(HN_WAVES * BH_WAVE) void head_norm_rope_write_kerne
 
 // proj [n_rows][row_stride]: a row holds, from `first`, H heads of q and G heads of k of `dim` and G heads of v of `vdim`;
 // bias f32 over those channels, or null; wq, wk f32 [dim], both or neither.  Pages as the attention kernels take them for G
-// kv heads of size `pad` (written when `write` is set); q_out [n_rows][H * pad].
+// kv heads of size `pad` (written when `write` is set); q_out [n_rows][H * pad].  `neighbours`: a turned pair is
+// dimensions 2i and 2i + 1 instead of i and i + turned/2; `magnitude` multiplies every cosine and sine.
 extern "C" int bh_head_norm_rope_write(const void* proj, int dtype, int row_stride, int first, const float* bias, const float* wq,
                                        const float* wk, float eps, const float* freq, int turned, const int32_t* positions,
                                        const int32_t* row_seq, void* q_out, void* k_pages, void* v_pages, const int32_t* page_table,
                                        int table_stride, int n_rows, int H, int G, int dim, int vdim, int pad, int kv_order, int write,
-                                       hipStream_t stream) {
+                                       int neighbours, float magnitude, hipStream_t stream) {
   BH_REQUIRE(n_rows > 0 && H > 0 && G > 0 && dim > 0 && vdim > 0, "head_norm_rope_write: sizes must be positive");
   BH_REQUIRE(pad >= dim && pad >= vdim, "head_norm_rope_write: heads of %d do not hold keys of %d and values of %d", pad, dim, vdim);
   BH_REQUIRE(turned >= 0 && turned % 2 == 0 && turned <= dim, "head_norm_rope_write: %d turned dimensions of %d", turned, dim);
@@ -111,7 +115,7 @@ extern "C" int bh_head_norm_rope_write(const void* proj, int dtype, int row_stri
   head_norm_rope_write_kernel<T><<<grid, HN_WAVES * BH_WAVE, lds, stream>>>((const T*)proj, row_stride, first, bias, wq, wk, eps, freq, \
                                                                            turned, positions, row_seq, (T*)q_out, (T*)k_pages,    \
                                                                            (T*)v_pages, page_table, table_stride, H, G, dim, vdim, \
-                                                                           pad, kv_order, write, per_group)
+                                                                           pad, kv_order, write, per_group, neighbours, magnitude)
   if (dtype == BH_F32) BH_HN(float);
   else if (dtype == BH_BF16) BH_HN(bf16_t);
   else return bh_fail("head_norm_rope_write: unknown dtype %d", dtype);

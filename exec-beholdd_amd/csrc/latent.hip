@@ -17,23 +17,25 @@ __global__ __launch_bounds__(256) void latent_write_kernel(
     const float* __restrict__ freq, int turned, const int32_t* __restrict__ positions, const int32_t* __restrict__ row_seq,
     T* __restrict__ k_pages, T* __restrict__ v_pages, const int32_t* __restrict__ page_table, int table_stride, int rank,
     int rot_dim, int kv_order, int write, T* __restrict__ query, long q_row, int q_head, int q_first, int src_head, int src_first,
-    int H) {
+    int H, const T* __restrict__ q_src, long q_src_row, int neighbours, float magnitude) {
   __shared__ float scratch[16];
   const int row = blockIdx.x;
   const T* x = down + (size_t)row * row_stride + offset;
   const int pos = positions[row], hd = rank + rot_dim;
   const int half = turned / 2;
-  if (query != nullptr) {      // the heads' rotated query parts, from the same projected row
+  if (query != nullptr) {      // the heads' rotated query parts, from the same projected row or from a matrix of their own
     for (int e = threadIdx.x; e < H * rot_dim; e += blockDim.x) {
       const int head = e / rot_dim, i = e % rot_dim;
-      const T* from = down + (size_t)row * row_stride + (size_t)head * src_head + src_first;
+      const T* from = q_src + (size_t)row * q_src_row + (size_t)head * src_head + src_first;
       float y;
       if (i < turned) {
-        const int pair = i < half ? i : i - half;
+        // the pair's first and second dimension: i and i + half, or the neighbours 2 pair and 2 pair + 1
+        const int pair = neighbours ? i / 2 : (i < half ? i : i - half);
+        const bool is_first = neighbours ? (i % 2 == 0) : (i < half);
         const float angle = (float)pos * freq[pair];
-        const float c = cosf(angle), s = sinf(angle);
-        const float u = to_f32(from[pair]), v = to_f32(from[pair + half]);
-        y = i < half ? u * c - v * s : v * c + u * s;
+        const float c = cosf(angle) * magnitude, s = sinf(angle) * magnitude;
+        const float u = to_f32(from[neighbours ? 2 * pair : pair]), v = to_f32(from[neighbours ? 2 * pair + 1 : pair + half]);
+        y = is_first ? u * c - v * s : v * c + u * s;
       } else {
         y = to_f32(from[i]);
       }
@@ -59,11 +61,12 @@ __global__ __launch_bounds__(256) void latent_write_kernel(
   for (int i = threadIdx.x; i < rot_dim; i += blockDim.x) {
     float y;
     if (i < turned) {
-      const int pair = i < half ? i : i - half;
+      const int pair = neighbours ? i / 2 : (i < half ? i : i - half);
+      const bool is_first = neighbours ? (i % 2 == 0) : (i < half);
       const float angle = (float)pos * freq[pair];
-      const float c = cosf(angle), s = sinf(angle);
-      const float u = to_f32(x[rank + pair]), v = to_f32(x[rank + pair + half]);
-      y = i < half ? u * c - v * s : v * c + u * s;
+      const float c = cosf(angle) * magnitude, s = sinf(angle) * magnitude;
+      const float u = to_f32(x[rank + (neighbours ? 2 * pair : pair)]), v = to_f32(x[rank + (neighbours ? 2 * pair + 1 : pair + half)]);
+      y = is_first ? u * c - v * s : v * c + u * s;
     } else {
       y = to_f32(x[rank + i]);
     }
@@ -75,15 +78,22 @@ __global__ __launch_bounds__(256) void latent_write_kernel(
 // down [n_rows][row_stride]: a row holds, from `offset`, rank latent elements and rot_dim key elements.
 // Pages as the attention kernels take them for one kv head of size rank + rot_dim (written when `write` is set).
 // With `query`, the same launch rotates the rot_dim elements at src_first of each of the H heads (src_head apart) of the
-// same row into query[row][head * q_head + q_first ..]: the heads' rotated query parts, beside the key's.
+// same row into query[row][head * q_head + q_first ..]: the heads' rotated query parts, beside the key's.  With `q_src`
+// (rows of q_src_row elements) the heads' parts are read from that matrix instead of `down`.  `neighbours`: a pair is
+// dimensions 2i and 2i + 1 instead of i and i + turned/2; `magnitude` multiplies every cosine and sine.
 extern "C" int bh_latent_write(const void* down, int dtype, int row_stride, int offset, const float* w, float eps,
                                const float* freq, int turned, const int32_t* positions, const int32_t* row_seq,
                                void* k_pages, void* v_pages, const int32_t* page_table, int table_stride, int n_rows,
                                int rank, int rot_dim, int kv_order, int write, void* query, long q_row, int q_head, int q_first,
-                               int src_head, int src_first, int H, hipStream_t stream) {
+                               int src_head, int src_first, int H, const void* q_src, long q_src_row, int neighbours,
+                               float magnitude, hipStream_t stream) {
   BH_REQUIRE(write || query != nullptr, "latent_write: nothing to do");
+  if (q_src == nullptr) {
+    q_src = down;
+    q_src_row = row_stride;
+  }
   BH_REQUIRE(query == nullptr || (H > 0 && q_first >= 0 && src_first >= 0 && q_first + rot_dim <= q_head && src_first + rot_dim <= src_head &&
-                                  (long)H * q_head <= q_row && H * src_head <= row_stride),
+                                  (long)H * q_head <= q_row && (long)H * src_head <= q_src_row),
              "latent_write: the heads' rotated slices do not lie inside their rows");
   BH_REQUIRE(n_rows > 0 && rank > 0 && rot_dim >= 0, "latent_write: sizes must be positive (the rotated part may be absent)");
   BH_REQUIRE(turned >= 0 && turned % 2 == 0 && turned <= rot_dim, "latent_write: %d turned dimensions of %d", turned, rot_dim);
@@ -95,7 +105,8 @@ extern "C" int bh_latent_write(const void* down, int dtype, int row_stride, int 
   latent_write_kernel<T><<<dim3(n_rows), dim3(256), 0, stream>>>((const T*)down, row_stride, offset, w, eps, freq, turned, \
                                                                  positions, row_seq, (T*)k_pages, (T*)v_pages, page_table, \
                                                                  table_stride, rank, rot_dim, kv_order, write, (T*)query, q_row, q_head, \
-                                                                 q_first, src_head, src_first, H)
+                                                                 q_first, src_head, src_first, H, (const T*)q_src, q_src_row, \
+                                                                 neighbours, magnitude)
   if (dtype == BH_F32) BH_LW(float);
   else if (dtype == BH_BF16) BH_LW(bf16_t);
   else return bh_fail("latent_write: unknown dtype %d", dtype);

@@ -276,3 +276,48 @@ extern "C" int bh_gelu_gate_table(const void* gate, int dtype, const int32_t* to
     return bh_fail("gelu_gate_table: unknown dtype %d", dtype);
   return bh_check_launch("gelu_gate_table");
 }
+
+// ---- a norm over a slice of wider rows, and a weighted sum of two matrices ---------------------------------------------
+//   slice_rmsnorm   out[row][i] = x[row][first + i] / sqrt(mean_i(x^2) + eps) * w[i] for i < width (x in the activations'
+//                   type, statistic and weight float32): a low-rank projection's share of a stacked product, normed
+//   weighted_sum    out = a x + b y, float32 (out may be x or y)
+template <typename T>
+__global__ __launch_bounds__(256) void slice_rmsnorm_kernel(const T* __restrict__ x, int row_stride, int first, const float* __restrict__ w,
+                                                            float eps, T* __restrict__ out, int width, int out_block_rows) {
+  __shared__ float scratch[8];
+  const int row = blockIdx.x;
+  const T* src = x + (size_t)row * row_stride + first;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    const float v = to_f32(src[i]);
+    ss += v * v;
+  }
+  const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / (float)width + eps);
+  for (int i = threadIdx.x; i < width; i += blockDim.x)
+    out[bh_rows_index(out_block_rows, row, i, width)] = from_f32<T>(to_f32(src[i]) * inv * (w ? w[i] : 1.f));
+}
+
+extern "C" int bh_slice_rmsnorm(const void* x, int dtype, int row_stride, int first, const float* w, float eps, void* out, int n_rows,
+                                int width, int out_block_rows, hipStream_t stream) {
+  BH_REQUIRE(n_rows > 0 && width > 0 && first >= 0 && first + width <= row_stride, "slice_rmsnorm: the slice lies outside a row of %d", row_stride);
+  BH_REQUIRE(out_block_rows == 0 || ((out_block_rows == 8 || out_block_rows == 16) && width % 32 == 0 && dtype == BH_BF16),
+             "slice_rmsnorm: rows in blocks of %d of width %d are not written", out_block_rows, width);
+  if (dtype == BH_F32)
+    slice_rmsnorm_kernel<float><<<n_rows, 256, 0, stream>>>((const float*)x, row_stride, first, w, eps, (float*)out, width, out_block_rows);
+  else if (dtype == BH_BF16)
+    slice_rmsnorm_kernel<bf16_t><<<n_rows, 256, 0, stream>>>((const bf16_t*)x, row_stride, first, w, eps, (bf16_t*)out, width, out_block_rows);
+  else
+    return bh_fail("slice_rmsnorm: unknown dtype %d", dtype);
+  return bh_check_launch("slice_rmsnorm");
+}
+
+__global__ __launch_bounds__(256) void weighted_sum_kernel(float* out, const float* x, float a, const float* y, float b, size_t n) {
+  for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (size_t)gridDim.x * blockDim.x) out[e] = a * x[e] + b * y[e];
+}
+
+extern "C" int bh_weighted_sum(float* out, const float* x, float a, const float* y, float b, long n, hipStream_t stream) {
+  BH_REQUIRE(n > 0, "weighted_sum: nothing to add");
+  const int blocks = (int)((n + 255) / 256 < 8192 ? (n + 255) / 256 : 8192);
+  weighted_sum_kernel<<<blocks, 256, 0, stream>>>(out, x, a, y, b, (size_t)n);
+  return bh_check_launch("weighted_sum");
+}

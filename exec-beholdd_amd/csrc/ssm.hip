@@ -2,7 +2,8 @@
 // recurrent state, and the gated norm behind it:
 //   ssm_scan            per (sequence, head): dt = softplus(dt_raw + dt_bias);  S <- exp(-exp(A_log) dt) S + dt B x^T;
 //                       y = S^T C + D x.   S is [N][vdim] float32 and lives in the sequence's state region.
-//   gated_group_rmsnorm out = rms_g(y * silu(z)) * w, the root mean square taken in `groups` equal parts of a row
+//   gated_group_rmsnorm out = rms_g(y * silu(z)) * w, the root mean square taken in `groups` equal parts of a row; with
+//                       `gate_after` the statistic is y's alone: out = rms_g(y) * w * silu(z)
 // Everything but the reading of dt_raw and z is float32.
 #include "common.h"
 
@@ -342,7 +343,8 @@ extern "C" int bh_ssm_scan_fast(const float* xbc, int xbc_stride, const void* pr
 template <typename T>
 __global__ __launch_bounds__(256) void gated_group_rmsnorm_kernel(const float* __restrict__ y, const T* __restrict__ z, int z_stride,
                                                                   int z_first, const float* __restrict__ w, float eps,
-                                                                  T* __restrict__ out, int width, int groups, int out_block_rows) {
+                                                                  T* __restrict__ out, int width, int groups, int out_block_rows,
+                                                                  int gate_after) {
   __shared__ float scratch[8];
   const int row = blockIdx.x, per = width / groups, c0 = blockIdx.y * per;
   const float* src = y + (size_t)row * width + c0;
@@ -350,19 +352,20 @@ __global__ __launch_bounds__(256) void gated_group_rmsnorm_kernel(const float* _
   float ss = 0.f;
   for (int i = threadIdx.x; i < per; i += blockDim.x) {
     const float g = to_f32(gate[i]);
-    const float v = src[i] * (g / (1.0f + expf(-g)));
+    const float v = gate_after ? src[i] : src[i] * (g / (1.0f + expf(-g)));
     ss += v * v;
   }
   const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / (float)per + eps);
   for (int i = threadIdx.x; i < per; i += blockDim.x) {
     const float g = to_f32(gate[i]);
-    const float v = src[i] * (g / (1.0f + expf(-g)));
+    const float v = src[i] * (g / (1.0f + expf(-g)));      // the gate's factor commutes with the norm's
     out[bh_rows_index(out_block_rows, row, c0 + i, width)] = from_f32<T>(v * inv * w[c0 + i]);
   }
 }
 
 extern "C" int bh_gated_group_rmsnorm(const float* y, const void* z, int dtype, int z_stride, int z_first, const float* w, float eps,
-                                      void* out, int n_rows, int width, int groups, int out_block_rows, hipStream_t stream) {
+                                      void* out, int n_rows, int width, int groups, int out_block_rows, int gate_after,
+                                      hipStream_t stream) {
   BH_REQUIRE(n_rows > 0 && width > 0 && groups > 0 && width % groups == 0, "gated_group_rmsnorm: %d columns in %d equal parts", width,
              groups);
   BH_REQUIRE(z_first >= 0 && z_first + width <= z_stride, "gated_group_rmsnorm: the gate lies outside its row");
@@ -371,10 +374,10 @@ extern "C" int bh_gated_group_rmsnorm(const float* y, const void* z, int dtype, 
   dim3 grid(n_rows, groups);
   if (dtype == BH_F32)
     gated_group_rmsnorm_kernel<float><<<grid, 256, 0, stream>>>(y, (const float*)z, z_stride, z_first, w, eps, (float*)out, width, groups,
-                                                                out_block_rows);
+                                                                out_block_rows, gate_after);
   else if (dtype == BH_BF16)
     gated_group_rmsnorm_kernel<bf16_t><<<grid, 256, 0, stream>>>(y, (const bf16_t*)z, z_stride, z_first, w, eps, (bf16_t*)out, width,
-                                                                 groups, out_block_rows);
+                                                                 groups, out_block_rows, gate_after);
   else
     return bh_fail("gated_group_rmsnorm: unknown dtype %d", dtype);
   return bh_check_launch("gated_group_rmsnorm");

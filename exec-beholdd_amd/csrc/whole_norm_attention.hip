@@ -7,7 +7,8 @@
 //                           pages of (sequence, position) as heads of `pad` (zeros beyond dim and vdim), so that keys of
 //                           one size and values of another go through kernels that know one head size
 //   conv_norm_rope_write    the same from the projected rows, the short convolution made on the way
-//   gate_heads              out[row][h][i] = attended[row][h][i] * sigmoid(gate[row][h][i]) for i < vdim
+//   gate_heads              out[row][h][i] = attended[row][h][i] * sigmoid(gate[row][h][i]) for i < vdim; the gate may be one
+//                           number a head (gate[row][h]) or absent (the heads' first vdim elements are put side by side)
 // Statistics, angles, cosines and sines are float32; the angle is the float32 product position * freq[i].
 #include "common.h"
 
@@ -230,31 +231,36 @@ extern "C" int bh_conv_norm_rope_write(const void* proj, int dtype, int row_stri
 template <typename T>
 __global__ __launch_bounds__(256) void gate_heads_kernel(const T* __restrict__ attended, int pad, const T* __restrict__ gate,
                                                          int gate_stride, int gate_first, T* __restrict__ out, int n_rows, int H,
-                                                         int vdim, int out_block_rows) {
+                                                         int vdim, int out_block_rows, int gate_per_head) {
   const int width = H * vdim;
   const size_t n = (size_t)n_rows * width;
   for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (size_t)gridDim.x * blockDim.x) {
     const int r = (int)(e / width), c = (int)(e % width), head = c / vdim, i = c % vdim;
     const float a = to_f32(attended[((size_t)r * H + head) * pad + i]);
-    const float g = to_f32(gate[(size_t)r * gate_stride + gate_first + c]);
+    if (gate == nullptr) {      // no gate: the heads' first vdim elements, side by side
+      out[bh_rows_index(out_block_rows, r, c, width)] = from_f32<T>(a);
+      continue;
+    }
+    const float g = to_f32(gate[(size_t)r * gate_stride + gate_first + (gate_per_head ? head : c)]);
     out[bh_rows_index(out_block_rows, r, c, width)] = from_f32<T>(a / (1.0f + expf(-g)));
   }
 }
 
 extern "C" int bh_gate_heads(const void* attended, int dtype, int pad, const void* gate, int gate_stride, int gate_first,
-                             void* out, int n_rows, int H, int vdim, int out_block_rows, hipStream_t stream) {
+                             void* out, int n_rows, int H, int vdim, int out_block_rows, int gate_per_head, hipStream_t stream) {
   BH_REQUIRE(n_rows > 0 && H > 0 && vdim > 0 && pad >= vdim, "gate_heads: sizes do not fit");
-  BH_REQUIRE(gate_first >= 0 && gate_first + H * vdim <= gate_stride, "gate_heads: the gate lies outside its row");
+  BH_REQUIRE(gate == nullptr || (gate_first >= 0 && gate_first + (gate_per_head ? H : H * vdim) <= gate_stride),
+             "gate_heads: the gate lies outside its row");
   BH_REQUIRE(out_block_rows == 0 || ((out_block_rows == 8 || out_block_rows == 16) && (H * vdim) % 32 == 0 && dtype == BH_BF16),
              "gate_heads: rows in blocks of %d of width %d are not written", out_block_rows, H * vdim);
   const size_t n = (size_t)n_rows * H * vdim;
   const int blocks = (int)((n + 255) / 256 < 8192 ? (n + 255) / 256 : 8192);
   if (dtype == BH_F32)
     gate_heads_kernel<float><<<blocks, 256, 0, stream>>>((const float*)attended, pad, (const float*)gate, gate_stride, gate_first,
-                                                       (float*)out, n_rows, H, vdim, out_block_rows);
+                                                       (float*)out, n_rows, H, vdim, out_block_rows, gate_per_head);
   else if (dtype == BH_BF16)
     gate_heads_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)attended, pad, (const bf16_t*)gate, gate_stride, gate_first,
-                                                        (bf16_t*)out, n_rows, H, vdim, out_block_rows);
+                                                        (bf16_t*)out, n_rows, H, vdim, out_block_rows, gate_per_head);
   else
     return bh_fail("gate_heads: unknown dtype %d", dtype);
   return bh_check_launch("gate_heads");

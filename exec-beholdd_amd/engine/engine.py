@@ -15,7 +15,7 @@ import torch
 
 from ..cache import SequenceCache
 from ..config.base import read_config_json
-from ..registry import resolve_architecture
+from ..registry import configuration_of, resolve_architecture
 from ..sampling import Sampler, SamplingParams
 from ..weights.binder import bind
 from ..weights.random_init import random_tensor_on_device
@@ -241,7 +241,7 @@ def open_model(model_dir: str, dtype, device):
     dtype = parse_dtype(dtype)
     data, path = read_config_json(model_dir)
     entry = resolve_architecture(data, path)
-    config = entry.config_class.from_dict(data, path)
+    config = configuration_of(entry, data, path, model_dir)
     model = entry.build(config)
     return model, bind(model.tensor_specs(), model_dir, dtype, device)
 
@@ -260,7 +260,7 @@ def random_model_on_device(config_dict: dict, seed: int, dtype, device):
     """A model with seeded random weights drawn on the device (nothing is written to disk)."""
     dtype = parse_dtype(dtype)
     entry = resolve_architecture(config_dict)
-    config = entry.config_class.from_dict(config_dict)
+    config = configuration_of(entry, config_dict)
     model = entry.build(config)
     specs = {spec.name: spec for spec in model.tensor_specs()}
     model.load(lambda name: random_tensor_on_device(specs[name], seed, device, dtype), device)

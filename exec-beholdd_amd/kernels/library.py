@@ -143,7 +143,7 @@ class KernelSizes:
             "bh_qk_norm_rope_cache_takes_sums": [i, i, i],
             "bh_gemm_bf16_bare_parts": [i, i, i, i],
             "bh_gemm_bf16_bare": [p, p, p, i, i, i, i, i, p],
-            "bh_attention_generic": [p, p, i, p, p, p, i, p, p, i, i, i, i, f, i, i, p],
+            "bh_attention_generic": [p, p, i, p, p, p, i, p, p, i, i, i, i, f, i, i, p, p],
             "bh_swiglu": [p, p, i, i, i, p],
             "bh_sample": [p, p, p, p, p, p, p, p, i, i, p],
             "bh_sample_scratch": [i, i],
@@ -154,7 +154,7 @@ class KernelSizes:
             "bh_gemm_bf16_then_norm": [p, p, p, i, i, i, i, p, i, f, p, p, i, i, p],
             "bh_rows_blocked": [p, p, i, i, i, i, p],
             "bh_gemm_bf16_finishes_norm": [i, i, i, i],
-            "bh_attention_bf16": [p, p, p, p, p, p, p, i, p, p, i, i, i, i, i, i, f, i, i, i, i, p],
+            "bh_attention_bf16": [p, p, p, p, p, p, p, i, p, p, i, i, i, i, i, i, f, i, i, i, i, p, p],
             "bh_attention_bf16_splits": [i, i, i, i, i],
             "bh_attention_bf16_writes_blocked": [i, i, i, i, i],
             "bh_attention_decode_fused": [p, p, p, p, p, p, p, i, p, p, i, i, i, i, f, i, i, i, p, p, i, f, p, p, i, i,
@@ -170,14 +170,14 @@ class KernelSizes:
             "bh_lightning_scan": [p, i, i, i, i, i, p, p, p, p, p, i, i, i, i, i, i, p, ctypes.c_long, p],
             "bh_lightning_chunks": [i, i, i, i, i, p],
             "bh_gated_rmsnorm": [p, p, i, i, p, p, i, i, f, i, p],
-            "bh_latent_write": [p, i, i, i, p, f, p, i, p, p, p, p, p, i, i, i, i, i, i, p, ctypes.c_long, i, i, i, i, i, p],
+            "bh_latent_write": [p, i, i, i, p, f, p, i, p, p, p, p, p, i, i, i, i, i, i, p, ctypes.c_long, i, i, i, i, i, p, ctypes.c_long, i, f, p],
             "bh_heads_linear": [p, ctypes.c_long, i, i, p, p, ctypes.c_long, i, i, i, i, i, i, i, i, p],
             "bh_rotate_heads": [p, ctypes.c_long, i, i, p, ctypes.c_long, i, i, i, p, i, p, i, i, i, p],
             "bh_layernorm": [p, p, p, p, p, i, i, i, f, i, p],
             "bh_cast_concat": [p, p, p, i, i, i, i, p],
             "bh_sum_layernorm": [p, p, f, p, p, p, i, i, i, f, i, p],
             "bh_gelu_tanh": [p, p, i, i, i, i, p],
-            "bh_head_norm_rope_write": [p, i, i, i, p, p, p, f, p, i, p, p, p, p, p, p, i, i, i, i, i, i, i, i, i, p],
+            "bh_head_norm_rope_write": [p, i, i, i, p, p, p, f, p, i, p, p, p, p, p, p, i, i, i, i, i, i, i, i, i, i, f, p],
             "bh_mlstm_gates": [p, p, f, p, ctypes.c_long, i, p, p, p, i, i, p],
             "bh_mlstm_scan": [p, i, i, i, i, i, p, p, ctypes.c_long, p, p, p, i, i, i, i, p],
             "bh_mlstm_finish": [p, p, p, i, i, i, p, f, p, i, i, i, i, p],
@@ -188,22 +188,25 @@ class KernelSizes:
             "bh_short_conv": [p, i, i, i, p, p, p, ctypes.c_long, p, p, p, p, i, i, i, i, p],
             "bh_short_conv_state": [p, i, i, i, p, ctypes.c_long, p, p, i, i, i, p],
             "bh_whole_norm_rope_write": [p, p, p, f, p, i, p, p, p, i, p, p, p, i, i, i, i, i, i, i, i, i, p],
-            "bh_gate_heads": [p, i, i, p, i, i, p, i, i, i, i, p],
+            "bh_gate_heads": [p, i, i, p, i, i, p, i, i, i, i, i, p],
             "bh_ssm_scan": [p, i, p, i, i, i, p, p, p, p, ctypes.c_long, p, p, p, i, i, i, i, i, p],
-            "bh_gated_group_rmsnorm": [p, p, i, i, i, p, f, p, i, i, i, i, p],
-            "bh_route_top_k": [p, p, p, p, i, i, i, p],
-            "bh_experts_gate_up": [p, i, p, p, p, i, i, i, i, f, f, p],
+            "bh_gated_group_rmsnorm": [p, p, i, i, i, p, f, p, i, i, i, i, i, p],
+            "bh_route_top_k": [p, p, p, p, i, i, i, i, p],
+            "bh_experts_gate_up": [p, i, p, p, p, i, i, i, i, f, f, f, p, p],
             "bh_experts_down": [p, i, p, p, p, p, i, i, i, i, p],
-            "bh_clamped_glu": [p, i, p, i, i, f, f, i, p],
+            "bh_clamped_glu": [p, i, p, i, i, f, f, i, f, p],
             "bh_conv_norm_rope_write": [p, i, i, i, p, i, p, ctypes.c_long, p, p, p, p, f, p, i, p, p, p, p, p, p, i, i, i, i, i, i, i, i, i, p],
             "bh_ssm_scan_fast": [p, i, p, i, i, i, p, p, p, p, ctypes.c_long, p, p, p, p, p, p, i, i, i, i, i, i, i, p],
             "bh_ssm_chunk_rows": [i, i, i],
             "bh_ssm_fast_takes": [i, i],
-            "bh_experts_products": [p, p, p, i, p, i, i, i, f, f, p],
+            "bh_experts_products": [p, p, p, i, p, i, i, i, f, f, f, p],
             "bh_experts_products_takes": [i, i],
             "bh_experts_group": [p, i, p, i, p, i, p],
-            "bh_experts_rows": [p, i, i, p, i, p, p, p, i, i, i, i, f, f, p],
-            "bh_experts_gather": [p, i, i, p, i, p, p, p, p, i, i, i, p],
+            "bh_experts_rows": [p, i, i, p, i, p, p, p, i, i, i, i, f, f, f, p, p],
+            "bh_experts_gather": [p, i, i, p, i, p, p, p, p, i, i, i, p, p],
+            "bh_gla_scan": [p, i, i, i, i, i, p, i, p, f, f, p, ctypes.c_long, p, p, p, i, i, i, i, p],
+            "bh_slice_rmsnorm": [p, i, i, i, p, f, p, i, i, i, p],
+            "bh_weighted_sum": [p, p, f, p, f, ctypes.c_long, p],
             "bh_experts_combine": [p, p, p, p, i, i, i, p],
         }
         for name, argtypes in table.items():
@@ -692,14 +695,17 @@ class HipKernels(KernelSizes):
             raise KernelError(f"{what}: the page table must be [sequences, pages]")
 
     def attention(self, q, out, k_pages, v_pages, page_table, row_seq, positions, n_heads, n_kv_heads, head_dim,
-                  scale, window=0, layout=None, chunk=0):
+                  scale, window=0, layout=None, chunk=0, sinks=None):
         """out[row, head] = softmax(q . K * scale) V over the keys of the row's sequence that the row
         may see: positions max(0, p - window + 1) .. p with a window, p - p % chunk .. p with chunks (counted from
         the sequence's position 0), else 0 .. p; not both.  `layout`, when given,
         says how rows group into sequences (seq_start int32 [n_seqs + 1] on the device, n_seqs,
         max_rows_per_seq, max_position), which the matrix-core kernel needs; rows of one sequence
-        are consecutive and in position order."""
+        are consecutive and in position order.  `sinks` (float32 [n_heads]): exp(sinks[head]) is one more term of the
+        head's softmax sums, with no key and no value."""
         n_rows = q.shape[0]
+        if sinks is not None and (sinks.shape != (n_heads,) or sinks.dtype != torch.float32):
+            raise KernelError(f"attention: one float32 sink a head ({n_heads}), got {tuple(sinks.shape)} of {sinks.dtype}")
         if window < 0 or chunk < 0 or (window and chunk):
             raise KernelError(f"attention: a window ({window}) or chunks ({chunk}) of a positive count of positions, not both")
         if chunk:
@@ -713,7 +719,7 @@ class HipKernels(KernelSizes):
                     int(layout.n_seqs), int(layout.max_rows_per_seq), n_heads, n_kv_heads, int(layout.max_position)))):
             rows_out = torch.empty(tuple(q.shape), dtype=q.dtype, device=self.device)   # this step's kernel writes rows
             self.attention(q, rows_out, k_pages, v_pages, page_table, row_seq, positions, n_heads, n_kv_heads, head_dim,
-                           scale, max(window, 0), layout, chunk)
+                           scale, max(window, 0), layout, chunk, sinks)
             self.to_blocked(rows_out, out)
             return
         if n_heads % n_kv_heads != 0:
@@ -741,14 +747,14 @@ class HipKernels(KernelSizes):
                              page_table.shape[1], self._ptr(positions, "positions", (torch.int32,)),
                              self._ptr(layout.seq_start, "seq_start", (torch.int32,)), n_seqs, n_rows, max_rows,
                              n_heads, n_kv_heads, head_dim, float(scale), int(window), int(layout.max_position),
-                             n_splits, _block_rows(out), self._stream()))
+                             n_splits, _block_rows(out), self._ptr(sinks, "sinks", (torch.float32,), True), self._stream()))
             return
         self._check(self.lib.bh_attention_generic(
             *common, _code(q, "q"), self._ptr(k_pages, "k_pages"), self._ptr(v_pages, "v_pages"),
             self._ptr(page_table, "page_table", (torch.int32,)), page_table.shape[1],
             self._ptr(row_seq, "row_seq", (torch.int32,)), self._ptr(positions, "positions", (torch.int32,)),
             n_rows, n_heads, n_kv_heads, head_dim, float(scale), int(window), self.kv_order(k_pages.dtype, head_dim),
-            self._stream()))
+            self._ptr(sinks, "sinks", (torch.float32,), True), self._stream()))
 
     def attention_decode_fused(self, qkv, out, q_weight, k_weight, eps, cos, sin, positions, k_pages, v_pages,
                                page_table, n_heads, n_kv_heads, head_dim, scale, window, write_kv, layout):
@@ -913,15 +919,57 @@ class HipKernels(KernelSizes):
             _code(proj, "gated_rmsnorm gate"), proj.shape[1], self._ptr(weight, "gated_rmsnorm weight", (torch.float32,), True),
             self._ptr(out, "gated_rmsnorm out"), n_rows, width, float(eps), _block_rows(out), self._stream()))
 
+    # ---- gated linear attention: a matrix state whose rows decay by factors that the token sets ----
+    def gla_scan(self, proj, q_off, k_off, v_off, z, bias, tau, q_scale, state, seq_start, seq_slot, out, n_heads, dim, vdim):
+        """Per (sequence, head): S <- diag(alpha_t) S + k_t v_t^T, out_t = S^T (q_scale q_t), alpha_t = sigmoid(z_t + bias)^(1/tau),
+        over the sequence's rows in order, from and into state[slot].  proj [n, P] holds q, k (H x dim) and v (H x vdim) from the
+        given columns; z f32 [n, H dim]; bias f32 [H dim]; state f32 [slots, H, dim, vdim]; out f32 [n, H vdim]."""
+        n_rows = proj.shape[0]
+        n_seqs = seq_slot.shape[0]
+        if tuple(out.shape) != (n_rows, n_heads * vdim) or z.shape != (n_rows, n_heads * dim) or bias.shape != (n_heads * dim,) \
+                or seq_start.shape != (n_seqs + 1,) or state.dim() != 4 or tuple(state.shape[1:]) != (n_heads, dim, vdim):
+            raise KernelError(f"gla_scan: shapes proj {tuple(proj.shape)}, z {tuple(z.shape)}, state {tuple(state.shape)}, "
+                              f"out {tuple(out.shape)} do not fit")
+        f32, i32 = (torch.float32,), (torch.int32,)
+        self._check(self.lib.bh_gla_scan(
+            self._ptr(proj, "gla_scan proj"), _code(proj, "gla_scan proj"), proj.shape[1], int(q_off), int(k_off), int(v_off),
+            self._ptr(z, "gla_scan decays", f32), z.shape[1], self._ptr(bias, "gla_scan bias", f32), float(tau), float(q_scale),
+            self._ptr(state, "gla_scan state", f32), n_heads * dim * vdim, self._ptr(seq_start, "seq_start", i32),
+            self._ptr(seq_slot, "seq_slot", i32), self._ptr(out, "gla_scan out", f32), n_seqs, n_heads, dim, vdim, self._stream()))
+
+    def slice_rmsnorm(self, x, first, weight, eps, out):
+        """out[r] = x[r, first : first + W] / sqrt(mean of its squares + eps) * weight; x [n, P] and out [n, W] (rows or
+        `BlockedRows`) in the activations' type, weight f32 [W]."""
+        n_rows, width = out.shape
+        if x.shape[0] != n_rows or first < 0 or first + width > x.shape[1] or out.dtype != x.dtype or weight.shape != (width,):
+            raise KernelError(f"slice_rmsnorm: shapes x {tuple(x.shape)}, out {tuple(out.shape)} do not fit")
+        self._check(self.lib.bh_slice_rmsnorm(
+            self._ptr(x, "slice_rmsnorm x"), _code(x, "slice_rmsnorm x"), x.shape[1], int(first),
+            self._ptr(weight, "slice_rmsnorm weight", (torch.float32,)), float(eps), self._ptr(out, "slice_rmsnorm out"), n_rows, width,
+            _block_rows(out), self._stream()))
+
+    def weighted_sum(self, out, x, a, y, b):
+        """out = a x + b y, float32 tensors of one shape (out may be x or y)."""
+        if x.shape != y.shape or out.shape != x.shape:
+            raise KernelError(f"weighted_sum: shapes {tuple(out.shape)}, {tuple(x.shape)}, {tuple(y.shape)} differ")
+        f32 = (torch.float32,)
+        self._check(self.lib.bh_weighted_sum(self._ptr(out, "weighted_sum out", f32), self._ptr(x, "weighted_sum x", f32), float(a),
+                                             self._ptr(y, "weighted_sum y", f32), float(b), x.numel(), self._stream()))
+
     # ---- attention over a cached latent ----
     def latent_write(self, down, offset, weight, eps, freq, turned, positions, row_seq, k_pages, v_pages, page_table,
-                     rank, rot_dim, write=True, query=None, query_head=0, query_first=0, source_head=0, source_first=0, n_heads=0):
+                     rank, rot_dim, write=True, query=None, query_head=0, query_first=0, source_head=0, source_first=0, n_heads=0,
+                     query_source=None, neighbours=False, magnitude=1.0):
         """From each row of `down` [n, P], at `offset`: c = RMSNorm(rank elements) * weight and the next rot_dim elements
         rotated (the first `turned` of them, pairs (i, i + turned/2), angle position * freq[i]); key [c | rotated] and
         value [c | 0] of ONE kv head of size rank + rot_dim go into the cache pages of (sequence, position) (unless
         `write` is False).  With `query` [n, >= n_heads * query_head] the same launch rotates the rot_dim elements at
-        `source_first` of each of the row's `n_heads` heads (`source_head` apart) into query[row, h * query_head + query_first ..]."""
+        `source_first` of each of the row's `n_heads` heads (`source_head` apart) into query[row, h * query_head + query_first ..];
+        the heads are those of `query_source` [n, >= n_heads * source_head] where one is given, else of `down`'s rows.
+        `neighbours`: a pair is dimensions (2i, 2i + 1) instead; `magnitude` multiplies every cosine and sine."""
         n_rows = down.shape[0]
+        if query_source is not None and (query_source.dim() != 2 or query_source.shape[0] != n_rows or query_source.dtype != down.dtype):
+            raise KernelError(f"latent_write: the queries' source {tuple(query_source.shape)} does not fit {n_rows} rows of {down.dtype}")
         head = rank + rot_dim
         if positions.shape != (n_rows,) or row_seq.shape != (n_rows,) or (weight is not None and tuple(weight.shape) != (rank,)) \
                 or (freq is not None and tuple(freq.shape) != (turned // 2,)):
@@ -937,7 +985,9 @@ class HipKernels(KernelSizes):
             self._ptr(k_pages, "k_pages"), self._ptr(v_pages, "v_pages"), self._ptr(page_table, "page_table", i32),
             page_table.shape[1], n_rows, int(rank), int(rot_dim), self.kv_order(k_pages.dtype, head), int(bool(write)),
             self._ptr(query, "rotated queries", None, True), query.shape[1] if query is not None else 0, int(query_head),
-            int(query_first), int(source_head), int(source_first), int(n_heads), self._stream()))
+            int(query_first), int(source_head), int(source_first), int(n_heads),
+            self._ptr(query_source, "queries' source", None, True), query_source.shape[1] if query_source is not None else 0,
+            int(bool(neighbours)), float(magnitude), self._stream()))
 
     def heads_linear(self, x, x_head, x_first, w, y, y_head, y_first, n_heads):
         """y[row, h, y_first + o] = sum_i w[h, i, o] * x[row, h, x_first + i]: x [n, >= H * x_head] and y [n, >= H * y_head]
@@ -999,10 +1049,12 @@ class HipKernels(KernelSizes):
                                           x.shape[0], x.shape[1], _block_rows(out), self._stream()))
 
     def head_norm_rope_write(self, proj, first, bias, q_weight, k_weight, eps, freq, turned, positions, row_seq, q_out, k_pages,
-                             v_pages, page_table, n_heads, n_kv_heads, dim, vdim, pad, write_kv):
+                             v_pages, page_table, n_heads, n_kv_heads, dim, vdim, pad, write_kv, neighbours=False,
+                             magnitude=1.0):
         """From column `first` of every row of `proj` [n, P]: q (H heads of dim), k (G of dim), v (G of vdim), plus `bias` (f32
         over those channels, or None); every head of q and k normed by its own root mean square times q_weight / k_weight
         (f32 [dim], both or None); dimensions i and i + turned/2 of every head of q and k turned by position * freq[i];
+        (`neighbours`: dimensions 2i and 2i + 1 instead; `magnitude` multiplies every cosine and sine);
         q -> q_out [n, H pad], k and v into the cache pages as heads of `pad` (see csrc/head_norm_attention.hip)."""
         n_rows = proj.shape[0]
         channels = (n_heads + n_kv_heads) * dim + n_kv_heads * vdim
@@ -1024,7 +1076,7 @@ class HipKernels(KernelSizes):
             self._ptr(freq, "frequencies", f32, True), int(turned), self._ptr(positions, "positions", i32),
             self._ptr(row_seq, "row_seq", i32), self._ptr(q_out, "q_out"), self._ptr(k_pages, "k_pages"), self._ptr(v_pages, "v_pages"),
             self._ptr(page_table, "page_table", i32), page_table.shape[1], n_rows, n_heads, n_kv_heads, dim, vdim, pad,
-            self.kv_order(k_pages.dtype, pad), int(bool(write_kv)), self._stream()))
+            self.kv_order(k_pages.dtype, pad), int(bool(write_kv)), int(bool(neighbours)), float(magnitude), self._stream()))
 
     # ---- a matrix memory with exponential gates, as a recurrence over a float32 state ----
     MLSTM_BESIDE = 4      # floats a row and head beside the read-out: a_t, b_t, m_t, n_t . q_t
@@ -1247,15 +1299,16 @@ class HipKernels(KernelSizes):
             self._ptr(page_table, "page_table", (torch.int32,)), page_table.shape[1], n_rows, n_heads, n_kv_heads, dim, vdim, pad,
             self.kv_order(k_pages.dtype, pad), int(bool(write_kv)), self._stream()))
 
-    def gate_heads(self, attended, pad, gate, gate_first, out, n_heads, vdim):
-        """out[r, h, i] = attended[r, h, i] * sigmoid(gate[r, gate_first + h vdim + i]), i < vdim; attended [n, H pad]."""
+    def gate_heads(self, attended, pad, gate, gate_first, out, n_heads, vdim, per_head=False):
+        """out[r, h, i] = attended[r, h, i] * sigmoid(gate[r, gate_first + h vdim + i]), i < vdim; attended [n, H pad].
+        `per_head`: one gate a head, gate[r, gate_first + h].  `gate` None: no gate, the heads' first vdim elements side by side."""
         n_rows = attended.shape[0]
-        if attended.shape != (n_rows, n_heads * pad) or tuple(out.shape) != (n_rows, n_heads * vdim) or gate.shape[0] != n_rows \
-                or gate.dtype != attended.dtype or out.dtype != attended.dtype:
+        if attended.shape != (n_rows, n_heads * pad) or tuple(out.shape) != (n_rows, n_heads * vdim) or (gate is not None and (gate.shape[0] != n_rows \
+                or gate.dtype != attended.dtype)) or out.dtype != attended.dtype:
             raise KernelError(f"gate_heads: shapes attended {tuple(attended.shape)}, out {tuple(out.shape)} do not fit")
         self._check(self.lib.bh_gate_heads(
-            self._ptr(attended, "gate_heads attended"), _code(attended, "gate_heads attended"), int(pad), self._ptr(gate, "gate_heads gate"),
-            gate.shape[1], int(gate_first), self._ptr(out, "gate_heads out"), n_rows, n_heads, vdim, _block_rows(out), self._stream()))
+            self._ptr(attended, "gate_heads attended"), _code(attended, "gate_heads attended"), int(pad), self._ptr(gate, "gate_heads gate", None, True),
+            gate.shape[1] if gate is not None else 0, int(gate_first), self._ptr(out, "gate_heads out"), n_rows, n_heads, vdim, _block_rows(out), int(bool(per_head)), self._stream()))
 
     # ---- a state-space recurrence with a scalar decay per head ----
     def ssm_scan(self, xbc, proj, dt_first, dt_bias, a_log, d_skip, state, state_offset, seq_start, seq_slot, out, n_heads, vdim,
@@ -1292,21 +1345,25 @@ class HipKernels(KernelSizes):
             *common, self._ptr(states, "chunk states", None, True), self._ptr(decays, "chunk decays", None, True),
             self._ptr(cum, "row decays", None, True), *rest, chunk_rows, chunks, self._stream()))
 
-    def gated_group_rmsnorm(self, y, z, z_first, weight, eps, out, groups):
+    def gated_group_rmsnorm(self, y, z, z_first, weight, eps, out, groups, gate_after=False):
         """out = rms_g(y * silu(z[:, z_first : z_first + W])) * weight, the root mean square over each of `groups` equal
-        parts of a row; y f32 [n, W], weight f32 [W], out [n, W] of z's type."""
+        parts of a row; y f32 [n, W], weight f32 [W], out [n, W] of z's type.
+        `gate_after`: the statistic is y's alone, out = rms_g(y) * weight * silu(z)."""
         n_rows, width = y.shape
         if tuple(out.shape) != (n_rows, width) or z.shape[0] != n_rows or weight.shape != (width,) or out.dtype != z.dtype:
             raise KernelError(f"gated_group_rmsnorm: shapes y {tuple(y.shape)}, z {tuple(z.shape)}, out {tuple(out.shape)} do not fit")
         self._check(self.lib.bh_gated_group_rmsnorm(
             self._ptr(y, "gated_group_rmsnorm y", (torch.float32,)), self._ptr(z, "gated_group_rmsnorm z"), _code(z, "gated_group_rmsnorm z"),
             z.shape[1], int(z_first), self._ptr(weight, "gated_group_rmsnorm weight", (torch.float32,)), float(eps),
-            self._ptr(out, "gated_group_rmsnorm out"), n_rows, width, int(groups), _block_rows(out), self._stream()))
+            self._ptr(out, "gated_group_rmsnorm out"), n_rows, width, int(groups), _block_rows(out), int(bool(gate_after)), self._stream()))
 
     # ---- routed experts ----
-    def route_top_k(self, logits, bias, chosen, weights):
+    def route_top_k(self, logits, bias, chosen, weights, scoring="softmax"):
         """chosen[r] = the `top` largest of logits[r] + bias (largest first, ties to the lower index), weights[r] = softmax over
-        those alone; logits f32 [n, E], chosen int32 [n, top], weights f32 [n, top]."""
+        those alone; logits f32 [n, E], chosen int32 [n, top], weights f32 [n, top].
+        `scoring` "sigmoid": weights[r] = the sigmoid of every chosen logit, each for itself."""
+        if scoring not in ("softmax", "sigmoid"):
+            raise KernelError(f"route_top_k: scoring is 'softmax' or 'sigmoid', got {scoring!r}")
         n_rows, experts = logits.shape
         top = chosen.shape[1]
         if chosen.shape != (n_rows, top) or weights.shape != (n_rows, top) or (bias is not None and bias.shape != (experts,)):
@@ -1314,10 +1371,11 @@ class HipKernels(KernelSizes):
         self._check(self.lib.bh_route_top_k(
             self._ptr(logits, "router logits", (torch.float32,)), self._ptr(bias, "router bias", (torch.float32,), True),
             self._ptr(chosen, "chosen", (torch.int32,)), self._ptr(weights, "route weights", (torch.float32,)), n_rows, experts, top,
-            self._stream()))
+            int(scoring == "sigmoid"), self._stream()))
 
-    def experts_gate_up(self, h, chosen, w_gate_up, inner, limit, alpha):
-        """inner[r * top + j] = act(Wg_e h[r], Wu_e h[r]) for e = chosen[r, j]; w_gate_up [E, 2 ff, K] (gate rows, then up rows)."""
+    def experts_gate_up(self, h, chosen, w_gate_up, inner, limit, alpha, shift=1.0, in_weights=None):
+        """inner[r * top + j] = act(Wg_e h[r], Wu_e h[r]) for e = chosen[r, j]; w_gate_up [E, 2 ff, K] (gate rows, then up rows).
+        `in_weights` float32 [n, top]: a pair's weight multiplies the expert's input (its gate and up sums)."""
         n_rows, k = h.shape
         top = chosen.shape[1]
         experts, twice, k_w = w_gate_up.shape
@@ -1327,18 +1385,19 @@ class HipKernels(KernelSizes):
             raise KernelError(f"experts_gate_up: shapes h {tuple(h.shape)}, weights {tuple(w_gate_up.shape)}, inner {tuple(inner.shape)} do not fit")
         self._check(self.lib.bh_experts_gate_up(
             self._ptr(h, "experts h"), _code(h, "experts h"), self._ptr(chosen, "chosen", (torch.int32,)), self._ptr(w_gate_up, "expert gate/up"),
-            self._ptr(inner, "experts inner"), n_rows, top, k, ff, float(limit), float(alpha), self._stream()))
+            self._ptr(inner, "experts inner"), n_rows, top, k, ff, float(limit), float(alpha), float(shift),
+            self._ptr(in_weights, "pair weights", (torch.float32,), True), self._stream()))
 
     def experts_down(self, inner, chosen, weights, w_down, hidden):
         """hidden[r] += sum_j weights[r, j] * Wd_e inner[r * top + j], e = chosen[r, j], j in order; w_down [E, D, ff]."""
         n_rows, top = chosen.shape
         experts, width, ff = w_down.shape
-        if tuple(inner.shape) != (n_rows * top, ff) or tuple(hidden.shape) != (n_rows, width) or weights.shape != (n_rows, top) \
+        if tuple(inner.shape) != (n_rows * top, ff) or tuple(hidden.shape) != (n_rows, width) or (weights is not None and weights.shape != (n_rows, top)) \
                 or w_down.dtype != inner.dtype:
             raise KernelError(f"experts_down: shapes inner {tuple(inner.shape)}, weights {tuple(w_down.shape)}, hidden {tuple(hidden.shape)} do not fit")
         self._check(self.lib.bh_experts_down(
             self._ptr(inner, "experts inner"), _code(inner, "experts inner"), self._ptr(chosen, "chosen", (torch.int32,)),
-            self._ptr(weights, "route weights", (torch.float32,)), self._ptr(w_down, "expert down"),
+            self._ptr(weights, "route weights", (torch.float32,), True), self._ptr(w_down, "expert down"),
             self._ptr(hidden, "experts hidden", (torch.float32,)), n_rows, top, ff, width, self._stream()))
 
     def experts_group(self, chosen, lists, counts):
@@ -1355,7 +1414,7 @@ class HipKernels(KernelSizes):
         """Whether `experts_rows` takes rows of that many inputs (16-byte loads)."""
         return inputs % 8 == 0
 
-    def experts_rows(self, rows, rows_per_pair_row, lists, counts, w, out, gated=False, limit=0.0, alpha=0.0):
+    def experts_rows(self, rows, rows_per_pair_row, lists, counts, w, out, gated=False, limit=0.0, alpha=0.0, shift=1.0, in_weights=None):
         """For every expert e and each of its pairs p (lists, counts): a product of w[e] with rows[p // rows_per_pair_row], the
         expert's matrix read once per workgroup.  gated: w [E, 2 N, K] (gate rows, then up rows), out [pairs, N] of the rows' type
         = act(gate, up); otherwise w [E, N, K] and out float32 [pairs, N]."""
@@ -1367,13 +1426,14 @@ class HipKernels(KernelSizes):
         self._check(self.lib.bh_experts_rows(
             self._ptr(rows, "experts rows"), _code(rows, "experts rows"), int(rows_per_pair_row), self._ptr(lists, "lists", (torch.int32,)),
             lists.shape[1], self._ptr(counts, "counts", (torch.int32,)), self._ptr(w, "expert weights"), self._ptr(out, "experts out"),
-            experts, k, n, int(bool(gated)), float(limit), float(alpha), self._stream()))
+            experts, k, n, int(bool(gated)), float(limit), float(alpha), float(shift),
+            self._ptr(in_weights, "pair weights", (torch.float32,), True), self._stream()))
 
     def experts_products_take(self, dtype, inputs: int, outputs: int) -> bool:
         """Whether `experts_products` takes products of these sizes and element type."""
         return dtype == torch.bfloat16 and bool(self.lib.bh_experts_products_takes(int(inputs), int(outputs)))
 
-    def experts_products(self, rows, w, tiles, out, gated=False, limit=0.0, alpha=0.0):
+    def experts_products(self, rows, w, tiles, out, gated=False, limit=0.0, alpha=0.0, shift=1.0):
         """All experts' products of a prompt in one launch on the matrix cores: rows bf16 [pairs, K] lie expert after expert,
         tiles int32 [n, 3] = (expert, first row, rows of the tile: 1 to 128) names every stretch; gated: w [E, 2 N, K] and out
         bf16 [pairs, N] = act(gate, up); otherwise w [E, N, K] and out float32 [pairs, N]."""
@@ -1385,11 +1445,11 @@ class HipKernels(KernelSizes):
         self._check(self.lib.bh_experts_products(
             self._ptr(rows, "experts rows", (torch.bfloat16,)), self._ptr(w, "expert weights", (torch.bfloat16,)),
             self._ptr(tiles, "tiles", (torch.int32,)), tiles.shape[0], self._ptr(out, "experts out"), k, n, int(bool(gated)), float(limit),
-            float(alpha), self._stream()))
+            float(alpha), float(shift), self._stream()))
 
-    def experts_gather(self, x, top, lists, counts, offsets, gathered, place):
+    def experts_gather(self, x, top, lists, counts, offsets, gathered, place, in_weights=None):
         """gathered[offsets[e] + i] = x[lists[e, i] // top] and place[lists[e, i]] = offsets[e] + i for i < counts[e]: the pairs'
-        input rows side by side, expert after expert."""
+        input rows side by side, expert after expert; with `in_weights` float32 [n, top] every copy times its pair's weight."""
         n_rows, k = x.shape
         experts = counts.shape[0]
         if tuple(gathered.shape) != (n_rows * top, k) or place.shape != (n_rows * top,) or offsets.shape != (experts,) \
@@ -1398,25 +1458,26 @@ class HipKernels(KernelSizes):
         self._check(self.lib.bh_experts_gather(
             self._ptr(x, "experts x"), _code(x, "experts x"), int(top), self._ptr(lists, "lists", (torch.int32,)), lists.shape[1],
             self._ptr(counts, "counts", (torch.int32,)), self._ptr(offsets, "offsets", (torch.int32,)), self._ptr(gathered, "gathered"),
-            self._ptr(place, "place", (torch.int32,)), experts, k, n_rows, self._stream()))
+            self._ptr(place, "place", (torch.int32,)), experts, k, n_rows,
+            self._ptr(in_weights, "pair weights", (torch.float32,), True), self._stream()))
 
-    def experts_combine(self, y, place, weights, hidden):
+    def experts_combine(self, y, place, weights, hidden, top=None):
         """hidden[r] += sum_j weights[r, j] * y[place[r * top + j]] (place None: y[r * top + j]), j in order; y f32 [pairs, D]."""
-        n_rows, top = weights.shape
+        n_rows, top = weights.shape if weights is not None else (hidden.shape[0], int(top))      # no weights: every share counts once
         if tuple(y.shape) != (n_rows * top, hidden.shape[1]) or hidden.shape[0] != n_rows or (place is not None and place.shape != (n_rows * top,)):
             raise KernelError(f"experts_combine: shapes y {tuple(y.shape)}, hidden {tuple(hidden.shape)} do not fit")
         self._check(self.lib.bh_experts_combine(
             self._ptr(y, "experts y", (torch.float32,)), self._ptr(place, "place", (torch.int32,), True),
-            self._ptr(weights, "route weights", (torch.float32,)), self._ptr(hidden, "experts hidden", (torch.float32,)), n_rows, top,
+            self._ptr(weights, "route weights", (torch.float32,), True), self._ptr(hidden, "experts hidden", (torch.float32,)), n_rows, top,
             hidden.shape[1], self._stream()))
 
-    def clamped_glu(self, gate_up, out, limit, alpha):
-        """out = g' * sigmoid(alpha g') * (u' + 1) with g' = min(g, limit), u' = clamp(u, -limit, limit); gate_up [n, 2 ff] = [g | u]."""
+    def clamped_glu(self, gate_up, out, limit, alpha, shift=1.0):
+        """out = g' * sigmoid(alpha g') * (u' + shift) with g' = min(g, limit), u' = clamp(u, -limit, limit); gate_up [n, 2 ff] = [g | u]."""
         n_rows, twice = gate_up.shape
         if tuple(out.shape) != (n_rows, twice // 2) or twice % 2 or out.dtype != gate_up.dtype:
             raise KernelError(f"clamped_glu: shapes gate_up {tuple(gate_up.shape)}, out {tuple(out.shape)} do not fit")
         self._check(self.lib.bh_clamped_glu(self._ptr(gate_up, "clamped_glu in"), _code(gate_up, "clamped_glu in"), self._ptr(out, "clamped_glu out"),
-                                            n_rows, twice // 2, float(limit), float(alpha), _block_rows(out), self._stream()))
+                                            n_rows, twice // 2, float(limit), float(alpha), _block_rows(out), float(shift), self._stream()))
 
     def stream_read(self, data, workgroups=256, nontemporal=True) -> int:
         """A yardstick, not a product path: read `data` (any contiguous tensor) once the way the streaming kernels

@@ -1,6 +1,6 @@
 """Models: the generic decoder and the architectures registered on it."""
 
 from .decoder import DecoderModel, build_decoder
-from . import qwen3, gokazen, pudorax, dupidra
+from . import qwen3, gokazen, pudorax, dupidra, vepelix
 
-__all__ = ["DecoderModel", "build_decoder", "qwen3", "gokazen", "pudorax", "dupidra"]
+__all__ = ["DecoderModel", "build_decoder", "qwen3", "gokazen", "pudorax", "dupidra", "vepelix"]

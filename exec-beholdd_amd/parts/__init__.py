@@ -15,10 +15,12 @@ from .embedding import CappedLMHead, Embedding, LMHead, ScaledEmbedding, ScaledL
 from .conv_attention import ConvGatedAttention
 from .state_space import StateSpaceScan
 from .experts import ClampedGLU, RoutedExperts
-from .token_side import LoopInput, TokenSideInput, TokenSideTable
+from .token_side import EmbeddingAgain, LoopInput, TokenSideInput, TokenSideTable
 from .gated_attention import GatedAttention
 from .mlstm import MatrixMemory
 from .post_norm import PostNormBlock
+from .gla import GatedLinearAttention
+from .parallel import ParallelMixers
 
 __all__ = ["BLOCKS", "FEED_FORWARDS", "MIXERS", "NORMS", "POSITION_ENCODINGS", "CacheNeed", "LayerCache",
            "Registry", "StepContext", "Linear", "RMSNorm", "NoPositionEncoding", "RotaryEncoding",

@@ -6,6 +6,12 @@
     expert(h) = Wd (g' * sigmoid(alpha g') * (u' + 1)),  g' = min(Wg h, limit),  u' = clamp(Wu h, -limit, limit)
     out = sum over chosen of weight * expert(h)  +  shared(h)        (the shared expert has the same form and runs for all)
 
+Variants, each a constructor parameter: `scoring="sigmoid"` weighs a chosen expert by the sigmoid of its own logit (no
+norming over the chosen); `weigh_input=True` puts the weight on the expert's input, out = sum expert(weight * h), which for
+these experts is a factor on the gate and up sums ahead of the activation (W (w h) = w (W h)); `limit`, `alpha` and `shift`
+shape the activation g' * sigmoid(alpha g') * (u' + shift), an infinite limit with alpha 1 and shift 0 being silu(g) * u; the
+shared expert is any feed-forward part.
+
 The experts' matrices are kept stacked: gate and up rows of an expert in one [2 ff, width] block, [experts, ...] in
 all.  The (row, choice) pairs are grouped by expert on the device (`experts_group`).  A step of few rows then runs a
 workgroup per expert and block of outputs that reads the expert's rows from memory once for all of its pairs
@@ -77,10 +83,14 @@ class RoutedExperts:
                               # one kernel reaches about 120 TFLOP/s whatever the size (tiles of 128 x 64 outputs re-read their
                               # operands through the L2), the products per expert cost about 25 us each and then run faster
 
-    def __init__(self, hidden: int, n_experts: int, top: int, ff: int, limit: float, prefix: str, shared: ClampedGLU | None = None,
-                 alpha: float = GATE_SLOPE, router_bias: bool = True):
+    def __init__(self, hidden: int, n_experts: int, top: int, ff: int, limit: float, prefix: str, shared=None,
+                 alpha: float = GATE_SLOPE, router_bias: bool = True, scoring: str = "softmax", weigh_input: bool = False,
+                 shift: float = 1.0):
         if not 1 <= top <= n_experts:
             raise ValueError(f"a row uses 1 to {n_experts} experts, got {top}")
+        if scoring not in ("softmax", "sigmoid"):
+            raise ValueError(f"experts are weighed by 'softmax' over the chosen or by each one's 'sigmoid', got {scoring!r}")
+        self.scoring, self.weigh_input, self.shift = scoring, bool(weigh_input), float(shift)
         self.hidden, self.n_experts, self.top, self.ff = int(hidden), int(n_experts), int(top), int(ff)
         self.limit, self.alpha, self.prefix, self.shared = float(limit), float(alpha), prefix, shared
         self.router = Linear(hidden, n_experts, prefix + "router")
@@ -138,24 +148,28 @@ class RoutedExperts:
         logits = self.router.forward(ctx, x, out_dtype=torch.float32)
         chosen = torch.empty((n, self.top), dtype=torch.int32, device=ctx.device)
         weights = ctx.new_f32(n, self.top)
-        k.route_top_k(logits, self.router_bias, chosen, weights)
+        k.route_top_k(logits, self.router_bias, chosen, weights, **({"scoring": self.scoring} if self.scoring != "softmax" else {}))
         ctx.extras["routing"] = (chosen, weights)
+        # where the weight goes: on the expert's input (the kernels that make gate and up take it) or on its output
+        act = {} if self.shift == 1.0 else {"shift": self.shift}
+        ahead = dict(act, in_weights=weights) if self.weigh_input else act
+        behind = None if self.weigh_input else weights
         pairs = n * self.top
         takes = getattr(k, "experts_rows_take", None)
         if takes is None or not (takes(self.hidden) and takes(self.ff)):
             inner = ctx.new_activations(pairs, self.ff)
-            k.experts_gate_up(x, chosen, self.w_gate_up, inner, self.limit, self.alpha)
-            k.experts_down(inner, chosen, weights, self.w_down, hidden)
+            k.experts_gate_up(x, chosen, self.w_gate_up, inner, self.limit, self.alpha, **ahead)
+            k.experts_down(inner, chosen, behind, self.w_down, hidden)
         else:
             lists = torch.empty((self.n_experts, n), dtype=torch.int32, device=ctx.device)
             counts = torch.empty((self.n_experts,), dtype=torch.int32, device=ctx.device)
             k.experts_group(chosen, lists, counts)
             if ctx.is_decode or pairs < self.PRODUCT_PAIRS * self.n_experts:
                 inner = ctx.new_activations(pairs, self.ff)
-                k.experts_rows(x, self.top, lists, counts, self.w_gate_up, inner, gated=True, limit=self.limit, alpha=self.alpha)
+                k.experts_rows(x, self.top, lists, counts, self.w_gate_up, inner, gated=True, limit=self.limit, alpha=self.alpha, **ahead)
                 y = ctx.new_f32(pairs, self.hidden)
                 k.experts_rows(inner, 1, lists, counts, self.w_down, y)
-                k.experts_combine(y, None, weights, hidden)
+                self._combine(k, y, None, behind, hidden)
             else:
                 self._as_products(ctx, x, lists, counts, weights, hidden)
         if self.shared is not None:
@@ -163,9 +177,17 @@ class RoutedExperts:
         return None
 
 
+    def _combine(self, k, y, place, weights, hidden):
+        if weights is not None:
+            k.experts_combine(y, place, weights, hidden)
+        else:
+            k.experts_combine(y, place, None, hidden, top=self.top)
+
     def _as_products(self, ctx, x, lists, counts, weights, hidden):
         """Every expert's pairs as one stretch of rows through the framework's matrix products."""
         k = ctx.kernels
+        act = {} if self.shift == 1.0 else {"shift": self.shift}
+        behind = None if self.weigh_input else weights
         n, pairs = x.shape[0], x.shape[0] * self.top
         matrices = self.for_products or [(self.w_gate_up[e], self.w_down[e]) for e in range(self.n_experts)]
         held = counts.cpu().tolist()              # the host waits for the routing here
@@ -176,27 +198,27 @@ class RoutedExperts:
         offsets = torch.tensor(starts, dtype=torch.int32, device=ctx.device)
         gathered = ctx.new_activations(pairs, self.hidden)
         place = torch.empty((pairs,), dtype=torch.int32, device=ctx.device)
-        k.experts_gather(x, self.top, lists, counts, offsets, gathered, place)
+        k.experts_gather(x, self.top, lists, counts, offsets, gathered, place, **({"in_weights": weights} if self.weigh_input else {}))
         if self.in_one_launch and 6.0 * pairs * self.ff * self.hidden <= self.ONE_LAUNCH_WORK:
             tiles = torch.tensor([(e, first + at, min(128, count - at)) for e, (first, count) in enumerate(zip(starts, held))
                                   for at in range(0, count, 128)], dtype=torch.int32, device=ctx.device)
             inner = ctx.new_activations(pairs, self.ff)
-            k.experts_products(gathered, self.w_gate_up, tiles, inner, gated=True, limit=self.limit, alpha=self.alpha)
+            k.experts_products(gathered, self.w_gate_up, tiles, inner, gated=True, limit=self.limit, alpha=self.alpha, **act)
             y = ctx.new_f32(pairs, self.hidden)
             k.experts_products(inner, self.w_down, tiles, y)
-            k.experts_combine(y, place, weights, hidden)
+            self._combine(k, y, place, behind, hidden)
             return
         both = ctx.new_activations(pairs, 2 * self.ff)
         for e, (first, count) in enumerate(zip(starts, held)):
             if count:
                 k.gemm(gathered[first:first + count], matrices[e][0], both[first:first + count])
         inner = ctx.new_activations(pairs, self.ff)
-        k.clamped_glu(both, inner, self.limit, self.alpha)
+        k.clamped_glu(both, inner, self.limit, self.alpha, **act)
         y = ctx.new_f32(pairs, self.hidden)
         for e, (first, count) in enumerate(zip(starts, held)):
             if count:
                 k.gemm(inner[first:first + count], matrices[e][1], y[first:first + count])
-        k.experts_combine(y, place, weights, hidden)
+        self._combine(k, y, place, behind, hidden)
 
 
 @FEED_FORWARDS.register("routed_experts")
@@ -205,3 +227,16 @@ def _build_routed_experts(config, layer_index, prefix, shared):
     common = ClampedGLU(config.hidden, sizes.shared.ff, sizes.shared.limit, prefix + "mlp.shared.") if sizes.shared is not None else None
     return RoutedExperts(config.hidden, sizes.experts, sizes.top, sizes.expert.ff, sizes.expert.limit, prefix + "mlp.", shared=common,
                          router_bias=getattr(sizes, "router_bias", True))
+
+
+@FEED_FORWARDS.register("routed_silu_experts")
+def _build_routed_silu_experts(config, layer_index, prefix, shared):
+    """Experts of the form Wd (silu(Wg h) * (Wu h)), each weighed by the sigmoid of its own router logit, the weight on the
+    expert's input; a shared expert of the same form."""
+    from .mlp import SwiGLU
+
+    sizes = config.layers[layer_index].mlp
+    names = ("gate", "up", "down")
+    common = SwiGLU(config.hidden, sizes.shared_ff, prefix + "mlp.shared.", names=names) if sizes.shared_ff else None
+    return RoutedExperts(config.hidden, sizes.experts, sizes.top, sizes.expert_ff, float("inf"), prefix + "mlp.", shared=common,
+                         alpha=1.0, router_bias=False, scoring="sigmoid", weigh_input=True, shift=0.0)

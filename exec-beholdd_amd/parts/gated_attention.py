@@ -13,7 +13,9 @@ keys and values written into the pages by one kernel (`head_norm_rope_write`).  
 values `vdim`; both are cached as heads of one padded size (zeros beyond), which the paged attention kernels take as it
 is.  Chunks are counted from a sequence's position 0, so what a row sees does not depend on how a prompt was cut; the
 cache keeps a chunk's (or a window's) span of positions and gives older pages back.  Norm statistics, angles and the
-softmax are float32.  Every size and constant is a constructor parameter; each mechanism can be switched off.
+softmax are float32.  Every size and constant is a constructor parameter; each mechanism can be switched off: without
+`gate` there is no Wg and the heads go to Wo as they are; `rotation` (a `RotaryFrequencies`) replaces `turned` and `base`
+where the frequencies are not the plain powers of the base; `neighbours` pairs dimensions 2i and 2i + 1.
 """
 
 from __future__ import annotations
@@ -34,12 +36,15 @@ class GatedAttention:
 
     def __init__(self, hidden: int, n_heads: int, n_kv_heads: int, dim: int, vdim: int, scale: float, prefix: str, *,
                  bias: bool = True, head_norm_eps: float | None = None, turned: int = 0, base: float = 10000.0,
-                 chunk: int = 0, window: int = 0):
+                 chunk: int = 0, window: int = 0, gate: bool = True, rotation: RotaryFrequencies | None = None,
+                 neighbours: bool = False):
         """`head_norm_eps` None: no query and key norms; `turned` 0: no rotation; `chunk` and `window` 0: every earlier key."""
         if n_heads % n_kv_heads:
             raise ValueError(f"{n_heads} query heads do not group evenly into {n_kv_heads} kv heads")
         if chunk and window:
             raise ValueError("keys are seen by chunk or by window, not both")
+        if rotation is not None:
+            turned = rotation.dims
         if turned % 2 or turned > dim:
             raise ValueError(f"the rotation turns pairs of a head's {dim} dimensions, got {turned}")
         self.hidden, self.n_heads, self.n_kv_heads, self.dim, self.vdim = int(hidden), int(n_heads), int(n_kv_heads), int(dim), int(vdim)
@@ -49,9 +54,10 @@ class GatedAttention:
         self.qkv_width = self.q_width + self.k_width + self.v_width
         self.gate_width = self.n_heads * self.vdim
         self.pad = padded_head(dim, vdim)
-        self.rotation = RotaryFrequencies(self.turned, base) if self.turned else None
-        self.proj = Linear(hidden, [self.q_width, self.k_width, self.v_width, self.gate_width],
-                           [prefix + "q", prefix + "k", prefix + "v", prefix + "g"])
+        self.gate, self.neighbours = bool(gate), bool(neighbours)
+        self.rotation = rotation if rotation is not None else (RotaryFrequencies(self.turned, base) if self.turned else None)
+        self.proj = Linear(hidden, [self.q_width, self.k_width, self.v_width] + ([self.gate_width] if self.gate else []),
+                           [prefix + "q", prefix + "k", prefix + "v"] + ([prefix + "g"] if self.gate else []))
         self.out = Linear(self.gate_width, hidden, prefix + "o")
         self.q_norm = self.k_norm = self.qkv_bias = None
 
@@ -99,14 +105,20 @@ class GatedAttention:
         proj = self.proj.forward(ctx, x)
         q = ctx.new_activations(n, self.n_heads * self.pad)
         freq = self.rotation.frequencies(ctx.device) if self.rotation is not None else None
+        turning = dict(neighbours=self.neighbours, magnitude=self.rotation.magnitude) if self.rotation is not None and (
+            self.neighbours or self.rotation.magnitude != 1.0) else {}
         k.head_norm_rope_write(proj, 0, self.qkv_bias, self.q_norm, self.k_norm, self.head_norm_eps or 0.0, freq, self.turned,
                                ctx.positions, ctx.row_seq, q, cache.k_pages, cache.v_pages, cache.page_table, self.n_heads,
-                               self.n_kv_heads, self.dim, self.vdim, self.pad, cache.writes)
-        attended = ctx.new_activations(n, self.n_heads * self.pad)
+                               self.n_kv_heads, self.dim, self.vdim, self.pad, cache.writes, **turning)
+        plain = not self.gate and self.pad == self.vdim      # the attended heads are the output projection's input as they are
+        attended = ctx.new_activations(n, self.n_heads * self.pad, reader=self.out.reader() if plain else None)
         k.attention(q, attended, cache.k_pages, cache.v_pages, cache.page_table, ctx.row_seq, ctx.positions, self.n_heads,
                     self.n_kv_heads, self.pad, self.scale, self.window, layout=ctx, chunk=self.chunk)
-        gated = ctx.new_activations(n, self.gate_width, reader=self.out.reader())
-        k.gate_heads(attended, self.pad, proj, self.qkv_width, gated, self.n_heads, self.vdim)
+        if plain:
+            gated = attended
+        else:
+            gated = ctx.new_activations(n, self.gate_width, reader=self.out.reader())
+            k.gate_heads(attended, self.pad, proj if self.gate else None, self.qkv_width, gated, self.n_heads, self.vdim)
         self.out.forward(ctx, gated, out=hidden, accumulate=not fresh)
         return None
 

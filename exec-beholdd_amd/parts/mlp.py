@@ -16,11 +16,11 @@ class SwiGLU:
     graph_safe_rows = None # ... whatever the number of tokens a sequence brings
     prepares_next_norm = True      # the down projection can carry the norm that follows
     takes_prepared_input = True    # x goes to the gate/up product untouched
-    def __init__(self, hidden: int, intermediate: int, prefix: str):
+    def __init__(self, hidden: int, intermediate: int, prefix: str, names=("gate_proj.weight", "up_proj.weight", "down_proj.weight")):
+        """`names`: what the gate, up and down matrices are called behind `prefix`."""
         self.hidden, self.intermediate = hidden, intermediate
-        self.gate_up = Linear(hidden, [intermediate, intermediate],
-                              [prefix + "gate_proj.weight", prefix + "up_proj.weight"])
-        self.down = Linear(intermediate, hidden, prefix + "down_proj.weight")
+        self.gate_up = Linear(hidden, [intermediate, intermediate], [prefix + names[0], prefix + names[1]])
+        self.down = Linear(intermediate, hidden, prefix + names[2])
 
     @property
     def input_reader(self):
@@ -115,3 +115,11 @@ def _build_squared_relu(config, layer_index, prefix, shared):
 @FEED_FORWARDS.register("none")
 def _build_no_feed_forward(config, layer_index, prefix, shared):
     return None
+
+
+@FEED_FORWARDS.register("clamped_glu")
+def _build_clamped_glu(config, layer_index, prefix, shared):
+    from .experts import ClampedGLU
+
+    sizes = config.layers[layer_index].mlp
+    return ClampedGLU(config.hidden, sizes.ff, sizes.limit, prefix + "mlp.")

@@ -10,6 +10,8 @@ kernel applies them.
 
 from __future__ import annotations
 
+import math
+
 import numpy as np
 import torch
 
@@ -48,20 +50,49 @@ class RotaryEncoding:
 class RotaryFrequencies:
     """The same rotation without a table: freq[i] = base^(-2i/dims) (computed in float64, kept as float32), and the
     kernel that rotates forms the angle position * freq[i] as a float32 product and takes its cosine and sine.
-    There is no longest position; `dims` of a vector's dimensions are turned, dimension i with i + dims/2."""
+    There is no longest position; `dims` of a vector's dimensions are turned, dimension i with i + dims/2, or, where the
+    mixer says so, the neighbours 2i and 2i + 1.
 
-    def __init__(self, dims: int, base: float):
+    `stretch` = (factor, original, fast, slow) slows the slow pairs down for contexts longer than `original` positions
+    (YaRN: B. Peng, J. Quesnelle, H. Fan, E. Shippole, "YaRN: Efficient Context Window Extension of Large Language
+    Models").  With d(t) = dims ln(original / (2 pi t)) / (2 ln base), the pair whose wave turns t times within
+    `original` positions, lo = max(floor(d(fast)), 0), hi = min(ceil(d(slow)), dims - 1) and
+    ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1):  freq_i <- freq_i / factor * ramp_i + freq_i (1 - ramp_i),
+    and every cosine and sine is multiplied by `magnitude` = 0.1 ln(factor) + 1 (1.0 without a stretch)."""
+
+    def __init__(self, dims: int, base: float, stretch=None):
         if dims <= 0 or dims % 2:
             raise ValueError(f"rotary width must be positive and even, got {dims}")
         if not (base > 0.0):
             raise ValueError(f"rotation base must be positive and finite, got {base}")
         self.dims, self.base = int(dims), float(base)
+        self.stretch, self.magnitude = None, 1.0
+        if stretch is not None:
+            factor, original, fast, slow = (float(value) for value in stretch)
+            if not (factor > 0.0 and original > 0.0 and fast > 0.0 and slow > 0.0) or base == 1.0:
+                raise ValueError(f"a stretch needs a positive factor, length and turn counts and a base other than 1, got {stretch!r}")
+            self.stretch = (factor, original, fast, slow)
+            self.magnitude = 0.1 * math.log(factor) + 1.0
         self._frequencies = None
+
+    def values(self) -> np.ndarray:
+        """The frequencies in float64, one per pair."""
+        plain = np.array([self.base ** (-2.0 * i / self.dims) for i in range(self.dims // 2)], dtype=np.float64)
+        if self.stretch is None:
+            return plain
+        factor, original, fast, slow = self.stretch
+
+        def pair_of(turns: float) -> float:
+            return self.dims * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(self.base))
+
+        low = max(math.floor(pair_of(fast)), 0)
+        high = min(math.ceil(pair_of(slow)), self.dims - 1)
+        ramp = np.clip((np.arange(self.dims // 2, dtype=np.float64) - low) / max(high - low, 0.001), 0.0, 1.0)
+        return plain / factor * ramp + plain * (1.0 - ramp)
 
     def frequencies(self, device) -> torch.Tensor:
         if self._frequencies is None or self._frequencies.device != torch.device(device):
-            values = np.array([self.base ** (-2.0 * i / self.dims) for i in range(self.dims // 2)], dtype=np.float64)
-            self._frequencies = torch.from_numpy(values.astype(np.float32)).to(device).contiguous()
+            self._frequencies = torch.from_numpy(self.values().astype(np.float32)).to(device).contiguous()
         return self._frequencies
 
 

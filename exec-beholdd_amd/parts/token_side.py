@@ -107,3 +107,25 @@ class LoopInput:
         both = ctx.new_activations(hidden.shape[0], 2 * self.hidden, reader=self.linear.reader())
         ctx.kernels.cast_concat(hidden, first, both)
         self.linear.forward(ctx, both, out=hidden)
+
+
+class EmbeddingAgain:
+    """The entry of a later pass of a looped stretch that adds the embedding's output to the residual: x <- x + x0, in
+    float32, x0 being what `keep` copied before the first layer changed the residual."""
+    graph_safe = True
+    graph_safe_rows = None
+
+    def tensor_specs(self):
+        return []
+
+    def load(self, get):
+        pass
+
+    def working_bytes(self, step) -> int:
+        return 0      # the copy has the residual's size, which the decoder counts once; this part does not know the width
+
+    def keep(self, ctx, hidden):
+        return hidden.clone()
+
+    def forward(self, ctx, hidden, first):
+        ctx.kernels.weighted_sum(hidden, hidden, 1.0, first, 1.0)

@@ -45,3 +45,23 @@ def resolve_architecture(config_dict: dict, origin: str = "config.json") -> Arch
         raise ConfigError(f"{origin}: unsupported architecture {name!r}; implemented architectures are "
                           + ", ".join(registered_architectures()))
     return entry
+
+
+def configuration_of(entry: ArchitectureEntry, config_dict: dict, origin: str = "config.json", model_dir=None):
+    """The architecture's typed configuration of a config.json.  A configuration class that says `needs_shapes` takes sizes
+    that only a tensor's shape gives from the checkpoint's header (name -> shape, no payload is read) as `shapes`; without a
+    model folder it gets None and has to find those sizes in the dictionary itself."""
+    if not getattr(entry.config_class, "needs_shapes", False):
+        return entry.config_class.from_dict(config_dict, origin)
+    shapes = None
+    if model_dir is not None:
+        import os
+
+        from .weights.safetensors_io import SafetensorsReader
+        if os.path.isdir(model_dir) and any(name.endswith(".safetensors") for name in os.listdir(model_dir)):
+            reader = SafetensorsReader(model_dir)
+            try:
+                shapes = {name: tuple(item.shape) for name, item in reader.entries.items()}
+            finally:
+                reader.close()
+    return entry.config_class.from_dict(config_dict, origin, shapes=shapes)

@@ -75,7 +75,7 @@ class TorchKernels:
             v_pages[page, :, :, pos % PAGE] = v[row].to(v_pages.dtype)
 
     def attention(self, q, out, k_pages, v_pages, page_table, row_seq, positions, n_heads, n_kv_heads, head_dim,
-                  scale, window=0, layout=None, chunk=0):
+                  scale, window=0, layout=None, chunk=0, sinks=None):
         self.calls.append("attention")
         assert not (window and chunk)
         n_rows = q.shape[0]
@@ -92,7 +92,10 @@ class TorchKernels:
             for head in range(n_heads):
                 kv = head // group
                 scores = (keys[:, kv, :].double() @ qh[row, head].double()).float() * scale
-                probs = torch.softmax(scores, dim=0)
+                if sinks is not None:      # one more term in the sum, with no value
+                    probs = torch.softmax(torch.cat([scores, sinks[head].float().reshape(1)]), dim=0)[:-1]
+                else:
+                    probs = torch.softmax(scores, dim=0)
                 result[row, head] = (probs.double() @ values[:, kv, :].double()).float()
         out.copy_(result.reshape(n_rows, n_heads * head_dim).to(out.dtype))
 
@@ -161,29 +164,41 @@ class TorchKernels:
 
     # ---- attention over a cached latent ----
     @staticmethod
-    def _turn(x, freq, turned, positions):
-        """x [n, ..., w]: the first `turned` of the last axis in pairs (i, i + turned/2) by the float32 angle position * freq[i]."""
+    def _turn(x, freq, turned, positions, neighbours=False, magnitude=1.0):
+        """x [n, ..., w]: the first `turned` of the last axis in pairs (i, i + turned/2), or (2i, 2i + 1) with `neighbours`, by the
+        float32 angle position * freq[i]; cosines and sines times `magnitude`."""
         if not turned:
             return x
         half = turned // 2
         angle = (positions.float()[:, None] * freq.float()[None, :]).double()
         shape = (x.shape[0],) + (1,) * (x.dim() - 2) + (half,)
-        c, s = torch.cos(angle).reshape(shape).float(), torch.sin(angle).reshape(shape).float()
+        c, s = (torch.cos(angle) * magnitude).reshape(shape).float(), (torch.sin(angle) * magnitude).reshape(shape).float()
+        if neighbours:
+            out = x.clone()
+            a, b = x[..., 0:turned:2], x[..., 1:turned:2]
+            out[..., 0:turned:2] = a * c - b * s
+            out[..., 1:turned:2] = b * c + a * s
+            return out
         a, b, rest = x[..., :half], x[..., half:turned], x[..., turned:]
         return torch.cat([a * c - b * s, b * c + a * s, rest], dim=-1)
 
     def latent_write(self, down, offset, weight, eps, freq, turned, positions, row_seq, k_pages, v_pages, page_table,
-                     rank, rot_dim, write=True, query=None, query_head=0, query_first=0, source_head=0, source_first=0, n_heads=0):
+                     rank, rot_dim, write=True, query=None, query_head=0, query_first=0, source_head=0, source_first=0, n_heads=0,
+                     query_source=None, neighbours=False, magnitude=1.0):
         self.calls.append("latent_write")
         if query is not None:
-            self.rotate_heads(down, source_head, source_first, query, query_head, query_first, freq, turned, positions, n_heads, rot_dim)
+            source = down if query_source is None else query_source
+            n = source.shape[0]
+            xs = source[:, :n_heads * source_head].float().reshape(n, n_heads, source_head)[:, :, source_first:source_first + rot_dim]
+            query[:, :n_heads * query_head].view(n, n_heads, query_head)[:, :, query_first:query_first + rot_dim] = self._turn(
+                xs, freq, turned, positions, neighbours, magnitude).to(query.dtype)
         if not write:
             return
         x = down[:, offset:offset + rank + rot_dim].float()
         c = x[:, :rank] * (1.0 / torch.sqrt((x[:, :rank].double() ** 2).mean(-1, keepdim=True) + eps)).float()
         if weight is not None:
             c = c * weight.float()
-        key = torch.cat([c, self._turn(x[:, rank:], freq, turned, positions)], dim=-1)
+        key = torch.cat([c, self._turn(x[:, rank:], freq, turned, positions, neighbours, magnitude)], dim=-1)
         value = torch.cat([c, torch.zeros(x.shape[0], rot_dim)], dim=-1)
         for row in range(x.shape[0]):
             pos = int(positions[row])
@@ -301,11 +316,16 @@ class TorchKernels:
             k_pages[page, :, pos % PAGE, :dim] = k[row].to(k_pages.dtype)
             v_pages[page, :, :vdim, pos % PAGE] = v[row].to(v_pages.dtype)
 
-    def gate_heads(self, attended, pad, gate, gate_first, out, n_heads, vdim):
+    def gate_heads(self, attended, pad, gate, gate_first, out, n_heads, vdim, per_head=False):
         self.calls.append("gate_heads")
         n = attended.shape[0]
-        a = attended.float().reshape(n, n_heads, pad)[..., :vdim].reshape(n, n_heads * vdim)
-        out.copy_((a * torch.sigmoid(gate[:, gate_first:gate_first + n_heads * vdim].float())).to(out.dtype))
+        a = attended.float().reshape(n, n_heads, pad)[..., :vdim]
+        if gate is None:
+            out.copy_(a.reshape(n, n_heads * vdim).to(out.dtype))
+        elif per_head:
+            out.copy_((a * torch.sigmoid(gate[:, gate_first:gate_first + n_heads].float())[:, :, None]).reshape(n, n_heads * vdim).to(out.dtype))
+        else:
+            out.copy_((a.reshape(n, n_heads * vdim) * torch.sigmoid(gate[:, gate_first:gate_first + n_heads * vdim].float())).to(out.dtype))
 
     # ---- norm behind the sum, GELU, heads normed one by one, a matrix memory ----
     def sum_layernorm(self, hidden, y, alpha, weight, bias, eps, rounded=None):
@@ -325,7 +345,7 @@ class TorchKernels:
         (x if out is None else out).copy_((0.5 * z * (1.0 + torch.tanh(0.7978845608028654 * (z + 0.044715 * z ** 3)))).to(x.dtype))
 
     def head_norm_rope_write(self, proj, first, bias, q_weight, k_weight, eps, freq, turned, positions, row_seq, q_out, k_pages,
-                             v_pages, page_table, n_heads, n_kv_heads, dim, vdim, pad, write_kv):
+                             v_pages, page_table, n_heads, n_kv_heads, dim, vdim, pad, write_kv, neighbours=False, magnitude=1.0):
         self.calls.append("head_norm_rope_write")
         n = proj.shape[0]
         q_width, k_width, v_width = n_heads * dim, n_kv_heads * dim, n_kv_heads * vdim
@@ -338,7 +358,7 @@ class TorchKernels:
         if q_weight is not None:
             rms = lambda t, w: (t.double() / torch.sqrt((t.double() ** 2).mean(-1, keepdim=True) + eps) * w.double()).float()
             q, k = rms(q, q_weight), rms(k, k_weight)
-        q, k = self._turn(q, freq, turned, positions), self._turn(k, freq, turned, positions)
+        q, k = self._turn(q, freq, turned, positions, neighbours, magnitude), self._turn(k, freq, turned, positions, neighbours, magnitude)
         wide = torch.zeros(n, n_heads, pad)
         wide[..., :dim] = q
         q_out.copy_(wide.reshape(n, n_heads * pad).to(q_out.dtype))
@@ -428,34 +448,38 @@ class TorchKernels:
                 out[row] = (torch.einsum("hnv,hn->hv", s, cm) + d_skip.double()[:, None] * x).float().reshape(-1)
             region[slot] = s.float().reshape(-1)
 
-    def gated_group_rmsnorm(self, y, z, z_first, weight, eps, out, groups):
+    def gated_group_rmsnorm(self, y, z, z_first, weight, eps, out, groups, gate_after=False):
         self.calls.append("gated_group_rmsnorm")
         n, width = y.shape
         g = z[:, z_first:z_first + width].double()
-        v = (y.double() * (g / (1 + torch.exp(-g)))).reshape(n, groups, width // groups)
+        gate = g / (1 + torch.exp(-g))
+        v = (y.double() if gate_after else y.double() * gate).reshape(n, groups, width // groups)
         v = (v / torch.sqrt((v ** 2).mean(-1, keepdim=True) + eps)).reshape(n, width)
-        out.copy_((v * weight.double()).to(out.dtype))
+        out.copy_((v * weight.double() * (gate if gate_after else 1.0)).to(out.dtype))
 
     # ---- routed experts ----
     @staticmethod
-    def _clamped_glu(g, u, limit, alpha):
+    def _clamped_glu(g, u, limit, alpha, shift=1.0):
         g, u = g.clamp(max=limit), u.clamp(min=-limit, max=limit)
-        return g * torch.sigmoid(alpha * g) * (u + 1.0)
+        return g * torch.sigmoid(alpha * g) * (u + shift)
 
-    def route_top_k(self, logits, bias, chosen, weights):
+    def route_top_k(self, logits, bias, chosen, weights, scoring="softmax"):
         self.calls.append("route_top_k")
         z = logits.double() + (bias.double() if bias is not None else 0.0)
         order = torch.argsort(-z, dim=-1, stable=True)[:, :chosen.shape[1]]
         chosen.copy_(order.to(torch.int32))
-        weights.copy_(torch.softmax(torch.gather(z, 1, order), dim=-1).float())
+        picked = torch.gather(z, 1, order)
+        weights.copy_((torch.sigmoid(picked) if scoring == "sigmoid" else torch.softmax(picked, dim=-1)).float())
 
-    def experts_gate_up(self, h, chosen, w_gate_up, inner, limit, alpha):
+    def experts_gate_up(self, h, chosen, w_gate_up, inner, limit, alpha, shift=1.0, in_weights=None):
         self.calls.append("experts_gate_up")
         top, ff = chosen.shape[1], w_gate_up.shape[1] // 2
         for row in range(h.shape[0]):
             for j in range(top):
                 both = w_gate_up[int(chosen[row, j])].double() @ h[row].double()
-                inner[row * top + j] = self._clamped_glu(both[:ff], both[ff:], limit, alpha).to(inner.dtype)
+                if in_weights is not None:
+                    both = both * float(in_weights[row, j])
+                inner[row * top + j] = self._clamped_glu(both[:ff], both[ff:], limit, alpha, shift).to(inner.dtype)
 
     def experts_down(self, inner, chosen, weights, w_down, hidden):
         self.calls.append("experts_down")
@@ -463,7 +487,7 @@ class TorchKernels:
         for row in range(hidden.shape[0]):
             total = torch.zeros(hidden.shape[1], dtype=torch.float64)
             for j in range(top):
-                total += float(weights[row, j]) * (w_down[int(chosen[row, j])].double() @ inner[row * top + j].double())
+                total += (float(weights[row, j]) if weights is not None else 1.0) * (w_down[int(chosen[row, j])].double() @ inner[row * top + j].double())
             hidden[row] += total.float()
 
     def experts_group(self, chosen, lists, counts):
@@ -477,33 +501,63 @@ class TorchKernels:
     def experts_rows_take(self, inputs):
         return inputs % 8 == 0
 
-    def experts_rows(self, rows, rows_per_pair_row, lists, counts, w, out, gated=False, limit=0.0, alpha=0.0):
+    def experts_rows(self, rows, rows_per_pair_row, lists, counts, w, out, gated=False, limit=0.0, alpha=0.0, shift=1.0, in_weights=None):
         self.calls.append("experts_rows")
         for e in range(counts.shape[0]):
             for pair in lists[e, :int(counts[e])].tolist():
                 result = w[e].double() @ rows[pair // rows_per_pair_row].double()
                 if gated:
                     half = result.shape[0] // 2
-                    result = self._clamped_glu(result[:half], result[half:], limit, alpha)
+                    if in_weights is not None:
+                        result = result * float(in_weights.reshape(-1)[pair])
+                    result = self._clamped_glu(result[:half], result[half:], limit, alpha, shift)
                 out[pair] = result.to(out.dtype)
 
-    def experts_gather(self, x, top, lists, counts, offsets, gathered, place):
+    def experts_gather(self, x, top, lists, counts, offsets, gathered, place, in_weights=None):
         self.calls.append("experts_gather")
         for e in range(counts.shape[0]):
             for i, pair in enumerate(lists[e, :int(counts[e])].tolist()):
-                gathered[int(offsets[e]) + i] = x[pair // top]
+                row = x[pair // top]
+                gathered[int(offsets[e]) + i] = row if in_weights is None else (row.float() * in_weights.reshape(-1)[pair]).to(x.dtype)
                 place[pair] = int(offsets[e]) + i
 
-    def experts_combine(self, y, place, weights, hidden):
+    def experts_combine(self, y, place, weights, hidden, top=None):
         self.calls.append("experts_combine")
-        n, top = weights.shape
+        n, top = weights.shape if weights is not None else (hidden.shape[0], int(top))
         index = (place if place is not None else torch.arange(n * top)).long().reshape(n, top)
-        hidden.add_((weights.double()[:, :, None] * y.double()[index]).sum(1).float())
+        share = weights.double()[:, :, None] if weights is not None else 1.0
+        hidden.add_((share * y.double()[index]).sum(1).float())
 
-    def clamped_glu(self, gate_up, out, limit, alpha):
+    def clamped_glu(self, gate_up, out, limit, alpha, shift=1.0):
         self.calls.append("clamped_glu")
         ff = out.shape[1]
-        out.copy_(self._clamped_glu(gate_up[:, :ff].double(), gate_up[:, ff:].double(), limit, alpha).to(out.dtype))
+        out.copy_(self._clamped_glu(gate_up[:, :ff].double(), gate_up[:, ff:].double(), limit, alpha, shift).to(out.dtype))
+
+    # ---- gated linear attention, a norm over a slice, a weighted sum ----
+    def gla_scan(self, proj, q_off, k_off, v_off, z, bias, tau, q_scale, state, seq_start, seq_slot, out, n_heads, dim, vdim):
+        self.calls.append("gla_scan")
+        kw, vw = n_heads * dim, n_heads * vdim
+        log_alpha = torch.nn.functional.logsigmoid(z.double() + bias.double()) / tau
+        for s in range(seq_slot.shape[0]):
+            slot = int(seq_slot[s])
+            memory = state[slot].double()
+            for row in range(int(seq_start[s]), int(seq_start[s + 1])):
+                q = proj[row, q_off:q_off + kw].double().reshape(n_heads, dim) * q_scale
+                key = proj[row, k_off:k_off + kw].double().reshape(n_heads, dim)
+                value = proj[row, v_off:v_off + vw].double().reshape(n_heads, vdim)
+                memory = torch.exp(log_alpha[row]).reshape(n_heads, dim, 1) * memory + key[:, :, None] * value[:, None, :]
+                memory = memory.float().double()      # the state is a float32
+                out[row] = torch.einsum("hdv,hd->hv", memory, q).float().reshape(-1)
+            state[slot] = memory.float()
+
+    def slice_rmsnorm(self, x, first, weight, eps, out):
+        self.calls.append("slice_rmsnorm")
+        v = x[:, first:first + out.shape[1]].double()
+        out.copy_((v / torch.sqrt((v ** 2).mean(-1, keepdim=True) + eps) * weight.double()).to(out.dtype))
+
+    def weighted_sum(self, out, x, a, y, b):
+        self.calls.append("weighted_sum")
+        out.copy_((a * x.double() + b * y.double()).float())
 
     def gemm_swiglu(self, a, w, out):
         self.calls.append("gemm_swiglu")
