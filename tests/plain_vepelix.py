@@ -249,3 +249,12 @@ def forward(config, w, tokens, residuals=None):
         if residuals is not None:
             residuals.append(x.copy())
     return linear(one_plus_norm(x, w["final.norm"], eps), w["head"])
+
+
+def greedy(config, w, prompt, n_new):
+    """The tokens that greedy decoding appends (ties to the lowest id), each from a whole forward of what stands so far."""
+    tokens, made = list(prompt), []
+    for _ in range(n_new):
+        made.append(int(np.argmax(forward(config, w, tokens)[-1])))
+        tokens.append(made[-1])
+    return made
