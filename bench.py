@@ -69,8 +69,15 @@ def parse():
                              "layers that run another layer's tensors) at layer sizes of real models beside Pudorax and Qwen3 at "
                              "equal width and as many layer runs: prefill and decode tokens per second, and every kernel of the "
                              "new design beside its like with the fraction of its roofline; prints one JSON line and exits")
+    parser.add_argument("--vepelix", action="store_true",
+                        help="the Vepelix design (attention over a cached latent with a query latent, sinks and a gate a head; "
+                             "windowed attention beside gated linear attention; experts weighed by sigmoid scores on their inputs; "
+                             "a looped stretch entered with the embedding's output) at layer sizes of real models beside Gokazen, "
+                             "Dupidra and Qwen3 at equal width and as many layer runs: prefill and decode tokens per second, and "
+                             "every kernel of the new design beside its like with the fraction of its roofline; prints one JSON "
+                             "line and exits")
     parser.add_argument("--alone", action="store_true",
-                        help="with --dupidra: the new design's two models only, without the models beside them and without the "
+                        help="with --dupidra or --vepelix: the new design's two models only, without the models beside them and without the "
                              "kernels timed alone (what a profiler should see of it)")
     parser.add_argument("--sampling", action="store_true",
                         help="time the selection kernel on 1, 8 and 64 rows of 151,936 logits (greedy, at a temperature, with "
@@ -818,6 +825,193 @@ def dupidra_bench(args, torch):
     return 0
 
 
+def vepelix_config(width, heads, vocab, experts=32, top=4, window=4096, rank=192, rot=64):
+    """Six layers of which two run twice (eight layer runs): attention over a latent of `rank` with a shared rotated key part of
+    `rot`, heads of 128 and queries through a latent of 3/8 of the width; windowed attention (heads of 128, four query heads to a
+    key/value head, a rotation over half a head) beside gated linear attention (keys of 64 and values of 128 a head, decays through
+    a rank of 16); `experts` experts of 3/8 of the width of which `top` are used and a shared one of 3/2 of the width in all layers
+    but the first, whose feed-forward is dense and three times the width."""
+    stretch = {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}
+    mlp = {"kind": "moe", "router": {"experts": experts, "top": top}, "expert": {"ff": 3 * width // 8}, "shared": {"ff": 3 * width // 2}}
+    latent = {"type": "latent_attention", "mlp": mlp,
+              "mixer": {"heads": heads, "dim": 128, "rot_dim": rot, "vdim": 128, "kv_rank": rank, "q_rank": 3 * width // 8,
+                        "scale": (128 + rot) ** -0.5, "rot": {"base": 500000.0, "dims": rot, "scaling": stretch}}}
+    side = {"type": "parallel", "mlp": mlp,
+            "mixer": {"left": {"heads": heads, "kv_heads": max(heads // 4, 1), "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                               "mask": {"size": window}, "rot": {"base": 1000000.0, "dims": 64, "scaling": stretch}},
+                      "right": {"heads": heads, "dim": 64, "vdim": 128, "tau": 16.0, "decay_rank": 16}, "left_scale": 1.0, "right_scale": 1.0}}
+    first = dict(latent, mlp={"kind": "dense", "ff": 3 * width, "limit": 7.0})
+    return {"architecture": "Vepelix", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "loop": {"start": 1, "stop": 3, "times": 2},
+            "layers": [first, latent, side, latent, side, latent]}
+
+
+def vepelix_kernels(K, torch, width, heads, context, rank=192, rot=64, window=4096):
+    """Every kernel that the design brought, and every older kernel in the turn the design gives it, beside its like among the
+    other models', alone, at a prompt of 2,048 rows and at a decode step of 8 rows over `context` cached tokens: microseconds and
+    the fraction of the roofline (the slower of its bytes at the HBM peak and its operations at the peak of the units it runs on)."""
+    from types import SimpleNamespace
+    bf16, dev = torch.bfloat16, "cuda:0"
+    dim = vdim = 128
+    page = K.page_size
+    out = {}
+
+    def note(name, us, n_bytes, flops=0.0, peak=PEAK_FLOPS["fp32"]):
+        floor = max(n_bytes / (PEAK_HBM_GBS * 1e9), flops / peak) * 1e6
+        out[name] = {"us": round(us, 1), "roofline_us": round(floor, 2), "fraction": round(floor / us, 3)}
+
+    def pages_for(n_seqs, length, kv_heads, head):
+        per = -(-length // page)
+        k_pages = torch.randn(n_seqs * per, kv_heads, page, head, device=dev).to(bf16)
+        v_pages = torch.randn(n_seqs * per, kv_heads, head, page, device=dev).to(bf16)
+        table = torch.arange(n_seqs * per, dtype=torch.int32, device=dev).view(n_seqs, per).contiguous()
+        return k_pages, v_pages, table
+
+    kv_heads = max(heads // 4, 1)
+    for rows, seqs, past, tag in ((2048, 1, 0, "prompt of 2,048"), (8, 8, context - 1, f"decode of 8 at {context}")):
+        each = rows // seqs
+        starts = torch.arange(0, rows + 1, each, dtype=torch.int32, device=dev)
+        slots = torch.arange(seqs, dtype=torch.int32, device=dev)
+        positions = (torch.arange(rows, dtype=torch.int32, device=dev) % each + past).contiguous()
+        row_seq = (torch.arange(rows, dtype=torch.int32, device=dev) // each).contiguous()
+        layout = SimpleNamespace(seq_start=starts, n_seqs=seqs, max_rows_per_seq=each, max_position=past + each - 1)
+        keys_seen = seqs * (past + each) if each == 1 else each * (each + 1) // 2
+        # -- gated linear attention (keys of 64, values of 128 a head) beside the linear attention with one decay a head
+        g_dim = 64
+        proj = torch.randn(rows, 2 * heads * g_dim + 2 * heads * vdim, device=dev).to(bf16)
+        decays = torch.randn(rows, heads * g_dim, device=dev)
+        bias = torch.full((heads * g_dim,), 4.0, device=dev)
+        state = torch.zeros(seqs, heads, g_dim, vdim, device=dev)
+        mixed = torch.empty(rows, heads * vdim, device=dev)
+        us = timed(lambda: K.gla_scan(proj, 0, heads * g_dim, 2 * heads * g_dim, decays, bias, 16.0, g_dim ** -0.5, state, starts, slots, mixed,
+                                      heads, g_dim, vdim), torch)
+        note(f"gla_scan, {tag}", us, 2 * state.numel() * 4 + rows * heads * (2 * g_dim + vdim) * 2 + decays.numel() * 4 + mixed.numel() * 4,
+             4.0 * rows * heads * g_dim * vdim)
+        l_proj = torch.randn(rows, 4 * heads * dim, device=dev).to(bf16)
+        l_state = torch.zeros(seqs, heads, dim, vdim, device=dev)
+        decay = torch.full((heads,), 0.99, device=dev)
+        us = timed(lambda: K.lightning_scan(l_proj, 0, heads * dim, 2 * heads * dim, l_state, decay, starts, slots, mixed, heads, dim, vdim), torch)
+        note(f"gokazen lightning_scan, {tag}", us, 2 * l_state.numel() * 4 + rows * 3 * heads * dim * 2 + mixed.numel() * 4, 4.0 * rows * heads * dim * vdim)
+        gated = torch.empty(rows, heads * vdim, device=dev, dtype=bf16)
+        weight = torch.ones(heads * vdim, device=dev)
+        us = timed(lambda: K.gated_group_rmsnorm(mixed, proj, 2 * heads * g_dim + heads * vdim, weight, 1e-6, gated, heads, gate_after=True), torch)
+        note(f"gated_group_rmsnorm with the gate behind the norm, {tag}", us, mixed.numel() * 4 + 2 * gated.numel() * 2)
+        us = timed(lambda: K.gated_rmsnorm(mixed, l_proj, 3 * heads * dim, weight, 1e-6, gated), torch)
+        note(f"gokazen gated_rmsnorm, {tag}", us, mixed.numel() * 4 + 2 * gated.numel() * 2)
+        # -- the weighted sum of the two mixers' results, beside the residual's update
+        a, b = torch.randn(rows, width, device=dev), torch.randn(rows, width, device=dev)
+        us = timed(lambda: K.weighted_sum(a, a, 1.2, b, 1.1), torch)
+        note(f"weighted_sum, {tag}", us, 3 * a.numel() * 4)
+        x, ones = torch.randn(rows, 1, width, device=dev), torch.ones(width, device=dev)
+        us = timed(lambda: K.streams_update(x, a, None, None, ones), torch)
+        note(f"gokazen streams_update (one stream), {tag}", us, 3 * a.numel() * 4)
+        # -- the latent layer: the query latent's norm, the cache write with stretched neighbour pairs, attention with sinks, the gate
+        q_rank, q_head, kv_head = 3 * width // 8, dim + rot, rank + rot
+        down = torch.randn(rows, q_rank + kv_head + heads, device=dev).to(bf16)
+        latent_q = torch.empty(rows, q_rank, device=dev, dtype=bf16)
+        rank_weight = torch.ones(q_rank, device=dev)
+        us = timed(lambda: K.slice_rmsnorm(down, 0, rank_weight, 1e-6, latent_q), torch)
+        note(f"slice_rmsnorm, {tag}", us, 2 * latent_q.numel() * 2)
+        hidden = torch.randn(rows, width, device=dev)
+        normed = torch.empty(rows, width, device=dev, dtype=bf16)
+        us = timed(lambda: K.rmsnorm(hidden, ones, 1e-6, normed), torch)
+        note(f"qwen3 rmsnorm, {tag}", us, hidden.numel() * 4 + normed.numel() * 2)
+        heads_rows = torch.randn(rows, heads * q_head, device=dev).to(bf16)
+        k_pages, v_pages, table = pages_for(seqs, past + each, 1, kv_head)
+        freq, latent_weight = torch.ones(rot // 2, device=dev), torch.ones(rank, device=dev)
+        query = torch.empty(rows, heads * kv_head, device=dev, dtype=bf16)
+        us = timed(lambda: K.latent_write(down, q_rank, latent_weight, 1e-6, freq, rot, positions, row_seq, k_pages, v_pages, table, rank, rot,
+                                          query=query, query_head=kv_head, query_first=rank, source_head=q_head, source_first=dim,
+                                          n_heads=heads, query_source=heads_rows, neighbours=True, magnitude=1.2), torch)
+        note(f"latent_write, neighbour pairs, queries from their own matrix, {tag}", us, rows * kv_head * 2 * 3 + 2 * rows * heads * rot * 2)
+        attended = torch.empty_like(query)
+        scale = (dim + rot) ** -0.5
+        sinks = torch.randn(heads, device=dev)
+        for name, kw in (("with sinks", dict(sinks=sinks)), ("gokazen, without", {})):
+            us = timed(lambda: K.attention(query, attended, k_pages, v_pages, table, row_seq, positions, heads, 1, kv_head, scale, 0,
+                                           layout=layout, **kw), torch)
+            note(f"attention over the latent ({heads} heads on one of {kv_head}) {name}, {tag}", us,
+                 2 * seqs * (past + each) * kv_head * 2 + 2 * query.numel() * 2, 4.0 * keys_seen * heads * kv_head, PEAK_FLOPS["bf16"])
+        values = torch.randn(rows, heads * vdim, device=dev).to(bf16)
+        gated_values = torch.empty_like(values)
+        us = timed(lambda: K.gate_heads(values, vdim, down, q_rank + kv_head, gated_values, heads, vdim, per_head=True), torch)
+        note(f"gate_heads, one gate a head, {tag}", us, 2 * values.numel() * 2)
+        wide_gate = torch.randn(rows, heads * vdim, device=dev).to(bf16)
+        us = timed(lambda: K.gate_heads(values, vdim, wide_gate, 0, gated_values, heads, vdim), torch)
+        note(f"pudorax gate_heads, one gate a value, {tag}", us, 3 * values.numel() * 2)
+        # -- the windowed attention: head norms, stretched neighbour pairs and the cache write; the attention within the window
+        q_w, k_w = heads * dim, kv_heads * dim
+        qkv = torch.randn(rows, q_w + 2 * k_w, device=dev).to(bf16)
+        head_weight, half_freq = torch.ones(dim, device=dev), torch.ones(32, device=dev)
+        wk, wv, wtable = pages_for(seqs, past + each, kv_heads, dim)
+        q_out = torch.empty(rows, heads * dim, device=dev, dtype=bf16)
+        for name, kw in (("neighbour pairs", dict(neighbours=True, magnitude=1.2)), ("dupidra, pairs half apart", {})):
+            us = timed(lambda: K.head_norm_rope_write(qkv, 0, None, head_weight, head_weight, 1e-6, half_freq, 64, positions, row_seq, q_out, wk, wv,
+                                                      wtable, heads, kv_heads, dim, dim, dim, True, **kw), torch)
+            note(f"head_norm_rope_write, {name}, {tag}", us, 2 * qkv.numel() * 2)
+        w_out = torch.empty_like(q_out)
+        seen = min(window, past + each)
+        us = timed(lambda: K.attention(q_out, w_out, wk, wv, wtable, row_seq, positions, heads, kv_heads, dim, dim ** -0.5, window, layout=layout), torch)
+        note(f"attention within a window of {window} ({heads} heads on {kv_heads} of {dim}), {tag}", us,
+             2 * seqs * seen * kv_heads * dim * 2 + 2 * q_out.numel() * 2, 4.0 * min(keys_seen, rows * seen) * heads * dim, PEAK_FLOPS["bf16"])
+        # -- routing by sigmoids, and the experts of a decode step with the weights on their inputs
+        experts, top, ff = 32, 4, 3 * width // 8
+        logits = torch.randn(rows, experts, device=dev)
+        chosen = torch.empty(rows, top, dtype=torch.int32, device=dev)
+        shares = torch.empty(rows, top, device=dev)
+        for name, kw in (("sigmoid scores", dict(scoring="sigmoid")), ("pudorax, softmax over the chosen", {})):
+            us = timed(lambda: K.route_top_k(logits, None, chosen, shares, **kw), torch)
+            note(f"route_top_k, {name}, {tag}", us, logits.numel() * 4 + 2 * chosen.numel() * 4)
+        if each == 1:
+            w_gu = torch.randn(experts, 2 * ff, width, device=dev).to(bf16) * 0.02
+            lists = torch.empty(experts, rows, dtype=torch.int32, device=dev)
+            counts = torch.empty(experts, dtype=torch.int32, device=dev)
+            K.experts_group(chosen, lists, counts)
+            active = int((counts > 0).sum())
+            x_rows = torch.randn(rows, width, device=dev).to(bf16)
+            inner = torch.empty(rows * top, ff, device=dev, dtype=bf16)
+            for name, kw in (("silu, weights on the inputs", dict(limit=float("inf"), alpha=1.0, shift=0.0, in_weights=shares)),
+                             ("pudorax, clamped, weights on the outputs", dict(limit=7.0, alpha=1.702))):
+                us = timed(lambda: K.experts_rows(x_rows, top, lists, counts, w_gu, inner, gated=True, **kw), torch)
+                note(f"experts_rows gate and up, {name}, {tag}", us, active * 2 * ff * width * 2)
+    return out
+
+
+def vepelix_bench(args, torch):
+    from beholdd.engine import Engine, random_model_on_device
+
+    device, points = "cuda:0", []
+    t = min(args.prefill_tokens, args.context)
+    for width, heads in ((2048, 16), (4096, 32)):
+        models = {"vepelix": vepelix_config(width, heads, 32768),
+                  "gokazen": gokazen_config(width, heads, 8, 3 * width, 32768),
+                  "dupidra": dupidra_config(width, heads, 32768),
+                  "qwen3": dict(QWEN3_8B, num_hidden_layers=8, hidden_size=width, num_attention_heads=heads,
+                                num_key_value_heads=heads // 4, intermediate_size=3 * width, vocab_size=32768)}
+        point = {"width": width, "heads": heads, "layer_runs": 8}
+        if args.alone:
+            models = {"vepelix": models["vepelix"]}
+        for name, config in models.items():
+            model = random_model_on_device(config, seed=0, dtype="bfloat16", device=device)
+            engine = Engine(model=model, dtype="bfloat16", max_tokens=args.batch * (-(-args.context // 64) * 64),
+                            max_slots=args.batch, device=device)
+            parameters = sum(int(np_prod(spec.shape)) for spec in model.tensor_specs())
+            seconds, _ = decode_run(engine, args.batch, args.context, args.steps, args.warmup, torch)
+            prefill = prefill_run(engine, t, torch)
+            point[name] = {"parameters": parameters, "decode_ms_per_step": round(seconds * 1e3, 4),
+                           "decode_tok_per_s": round(args.batch / seconds, 1), "prefill_ms": round(prefill * 1e3, 3),
+                           "prefill_tok_per_s": round(t / prefill, 1)}
+            kernels = engine.kernels
+            del engine, model
+            torch.cuda.empty_cache()
+        points.append(point)
+    line = {"metric": f"Vepelix beside Gokazen, Dupidra and Qwen3 at equal width and as many layer runs: decode tok/s @ batch {args.batch}, context {args.context}; prefill of {t} tokens",
+            "unit": "tok/s", "value": points[-1]["vepelix"]["decode_tok_per_s"], "dtype": "bf16", "data": "synthetic", "n_gpus": 1,
+            "steps": args.steps, "warmup": args.warmup, "higher_is_better": True, "points": points,
+            "kernels": {} if args.alone else vepelix_kernels(kernels, torch, 4096, 32, args.context)}
+    print(json.dumps(line))
+    return 0
+
+
 def np_prod(shape):
     total = 1
     for axis in shape:
@@ -843,6 +1037,8 @@ def main():
         return pudorax_bench(args, torch)
     if args.dupidra:
         return dupidra_bench(args, torch)
+    if args.vepelix:
+        return vepelix_bench(args, torch)
 
     from beholdd.engine import Engine, random_model_on_device
 
