@@ -363,6 +363,40 @@ __global__ __launch_bounds__(256) void gated_group_rmsnorm_kernel(const float* _
   }
 }
 
+// The same with a wave a group, for groups of up to 512 elements (the heads of a row normed one by one): a workgroup takes a
+// row, its four waves the row's groups in turn, a lane keeps its elements in registers between the statistic and the write.
+template <typename T>
+__global__ __launch_bounds__(256) void gated_group_rmsnorm_waves_kernel(const float* __restrict__ y, const T* __restrict__ z, int z_stride,
+                                                                        int z_first, const float* __restrict__ w, float eps,
+                                                                        T* __restrict__ out, int width, int groups, int out_block_rows,
+                                                                        int gate_after) {
+  const int row = blockIdx.x, per = width / groups, lane = threadIdx.x % BH_WAVE;
+  for (int group = threadIdx.x / BH_WAVE; group < groups; group += 4) {
+    const int c0 = group * per;
+    const float* src = y + (size_t)row * width + c0;
+    const T* gate = z + (size_t)row * z_stride + z_first + c0;
+    float held[8], gates[8];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int c = lane + i * BH_WAVE;
+      held[i] = gates[i] = 0.f;
+      if (c < per) {
+        const float g = to_f32(gate[c]);
+        gates[i] = g / (1.0f + expf(-g));
+        held[i] = gate_after ? src[c] : src[c] * gates[i];
+        ss += held[i] * held[i];
+      }
+    }
+    const float inv = 1.0f / sqrtf(wave_sum(ss) / (float)per + eps);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int c = lane + i * BH_WAVE;
+      if (c < per) out[bh_rows_index(out_block_rows, row, c0 + c, width)] = from_f32<T>(held[i] * (gate_after ? gates[i] : 1.0f) * inv * w[c0 + c]);
+    }
+  }
+}
+
 extern "C" int bh_gated_group_rmsnorm(const float* y, const void* z, int dtype, int z_stride, int z_first, const float* w, float eps,
                                       void* out, int n_rows, int width, int groups, int out_block_rows, int gate_after,
                                       hipStream_t stream) {
@@ -372,6 +406,17 @@ extern "C" int bh_gated_group_rmsnorm(const float* y, const void* z, int dtype, 
   BH_REQUIRE(out_block_rows == 0 || ((out_block_rows == 8 || out_block_rows == 16) && width % 32 == 0 && dtype == BH_BF16),
              "gated_group_rmsnorm: rows in blocks of %d of width %d are not written", out_block_rows, width);
   dim3 grid(n_rows, groups);
+  if (groups > 1 && width / groups <= 8 * BH_WAVE && n_rows >= bh_compute_units() / 2) {      // many rows of small groups: a wave a group
+    if (dtype == BH_F32)
+      gated_group_rmsnorm_waves_kernel<float><<<n_rows, 256, 0, stream>>>(y, (const float*)z, z_stride, z_first, w, eps, (float*)out, width,
+                                                                          groups, out_block_rows, gate_after);
+    else if (dtype == BH_BF16)
+      gated_group_rmsnorm_waves_kernel<bf16_t><<<n_rows, 256, 0, stream>>>(y, (const bf16_t*)z, z_stride, z_first, w, eps, (bf16_t*)out, width,
+                                                                           groups, out_block_rows, gate_after);
+    else
+      return bh_fail("gated_group_rmsnorm: unknown dtype %d", dtype);
+    return bh_check_launch("gated_group_rmsnorm");
+  }
   if (dtype == BH_F32)
     gated_group_rmsnorm_kernel<float><<<grid, 256, 0, stream>>>(y, (const float*)z, z_stride, z_first, w, eps, (float*)out, width, groups,
                                                                 out_block_rows, gate_after);
