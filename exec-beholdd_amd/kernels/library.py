@@ -204,7 +204,8 @@ class KernelSizes:
             "bh_experts_group": [p, i, p, i, p, i, p],
             "bh_experts_rows": [p, i, i, p, i, p, p, p, i, i, i, i, f, f, f, p, p],
             "bh_experts_gather": [p, i, i, p, i, p, p, p, p, i, i, i, p, p],
-            "bh_gla_scan": [p, i, i, i, i, i, p, i, p, f, f, p, ctypes.c_long, p, p, p, i, i, i, i, p],
+            "bh_gla_scan": [p, i, i, i, i, i, p, i, p, f, f, p, ctypes.c_long, p, p, p, i, i, i, i, i, i, i, p, p],
+            "bh_gla_chunk_rows": [i, i, i, i, i],
             "bh_slice_rmsnorm": [p, i, i, i, p, f, p, i, i, i, p],
             "bh_weighted_sum": [p, p, f, p, f, ctypes.c_long, p],
             "bh_experts_combine": [p, p, p, p, i, i, i, p],
@@ -274,6 +275,14 @@ class KernelSizes:
             return 0
         return (_rounded(n_seqs * chunks * n_heads * n_state * vdim * 4) + _rounded(n_seqs * chunks * n_heads * 4)
                 + _rounded(n_rows * n_heads * 4))
+
+    def gla_chunk_bytes(self, n_seqs, n_rows, max_rows, n_heads, dim, vdim) -> int:
+        """Bytes of scratch memory that `gla_scan` allocates for a step of these sizes (long sequences cut into chunks)."""
+        chunk_rows = int(self.lib.bh_gla_chunk_rows(int(n_seqs), int(max_rows), int(n_heads), int(dim), int(vdim)))
+        if chunk_rows >= max_rows:
+            return 0
+        chunks = -(-int(max_rows) // chunk_rows)
+        return _rounded((n_seqs * chunks * n_heads * dim * (vdim + 1) + n_rows * n_heads * dim) * 4)
 
     def packs(self, rows, cols, act_size) -> bool:
         """Whether `pack_weight` regroups a matrix of this shape and element size."""
@@ -920,12 +929,21 @@ class HipKernels(KernelSizes):
             self._ptr(out, "gated_rmsnorm out"), n_rows, width, float(eps), _block_rows(out), self._stream()))
 
     # ---- gated linear attention: a matrix state whose rows decay by factors that the token sets ----
-    def gla_scan(self, proj, q_off, k_off, v_off, z, bias, tau, q_scale, state, seq_start, seq_slot, out, n_heads, dim, vdim):
+    def gla_scan(self, proj, q_off, k_off, v_off, z, bias, tau, q_scale, state, seq_start, seq_slot, out, n_heads, dim, vdim,
+                 max_rows_per_seq=None):
         """Per (sequence, head): S <- diag(alpha_t) S + k_t v_t^T, out_t = S^T (q_scale q_t), alpha_t = sigmoid(z_t + bias)^(1/tau),
         over the sequence's rows in order, from and into state[slot].  proj [n, P] holds q, k (H x dim) and v (H x vdim) from the
-        given columns; z f32 [n, H dim]; bias f32 [H dim]; state f32 [slots, H, dim, vdim]; out f32 [n, H vdim]."""
+        given columns; z f32 [n, H dim]; bias f32 [H dim]; state f32 [slots, H, dim, vdim]; out f32 [n, H vdim].
+        `max_rows_per_seq` (the rows of the step's longest sequence; all rows where it is not said) lets long sequences be walked
+        in chunks side by side, with scratch memory for this call."""
         n_rows = proj.shape[0]
         n_seqs = seq_slot.shape[0]
+        most = int(max_rows_per_seq) if max_rows_per_seq else n_rows
+        chunk_rows = int(self.lib.bh_gla_chunk_rows(n_seqs, most, n_heads, dim, vdim))
+        scratch = None
+        if chunk_rows < most:
+            chunks = -(-most // chunk_rows)
+            scratch = torch.empty(n_seqs * chunks * n_heads * dim * (vdim + 1) + n_rows * n_heads * dim, dtype=torch.float32, device=self.device)
         if tuple(out.shape) != (n_rows, n_heads * vdim) or z.shape != (n_rows, n_heads * dim) or bias.shape != (n_heads * dim,) \
                 or seq_start.shape != (n_seqs + 1,) or state.dim() != 4 or tuple(state.shape[1:]) != (n_heads, dim, vdim):
             raise KernelError(f"gla_scan: shapes proj {tuple(proj.shape)}, z {tuple(z.shape)}, state {tuple(state.shape)}, "
@@ -935,7 +953,8 @@ class HipKernels(KernelSizes):
             self._ptr(proj, "gla_scan proj"), _code(proj, "gla_scan proj"), proj.shape[1], int(q_off), int(k_off), int(v_off),
             self._ptr(z, "gla_scan decays", f32), z.shape[1], self._ptr(bias, "gla_scan bias", f32), float(tau), float(q_scale),
             self._ptr(state, "gla_scan state", f32), n_heads * dim * vdim, self._ptr(seq_start, "seq_start", i32),
-            self._ptr(seq_slot, "seq_slot", i32), self._ptr(out, "gla_scan out", f32), n_seqs, n_heads, dim, vdim, self._stream()))
+            self._ptr(seq_slot, "seq_slot", i32), self._ptr(out, "gla_scan out", f32), n_seqs, n_heads, dim, vdim, n_rows, most,
+            chunk_rows, self._ptr(scratch, "gla_scan scratch", f32, True), self._stream()))
 
     def slice_rmsnorm(self, x, first, weight, eps, out):
         """out[r] = x[r, first : first + W] / sqrt(mean of its squares + eps) * weight; x [n, P] and out [n, W] (rows or

@@ -11,8 +11,9 @@ Hardware-Efficient Training".)  q, k, v and g are one stacked product; the decay
 product of the low-rank rows.  The state is a fixed-size float32 region of the cache (kind "state"): a step continues from
 what the sequence's slot holds, whatever the step's cut, and a slot starts at zero.  The decays (through the logarithm of
 the sigmoid), the state and both products of the recurrence are float32; the projections have the engine's activation
-type.  One kernel walks a sequence's rows of the step in order (`gla_scan`, prompts and decode steps alike), one norms
-and gates (`gated_group_rmsnorm` with the gate behind the norm).  Every size and constant is a constructor parameter.
+type.  One kernel walks a sequence's rows of the step in order (`gla_scan`, prompts and decode steps alike; long
+sequences in chunks side by side, after which the chunks' states are joined in order and every chunk's rows get what they owe
+the state their chunk started from), one norms and gates (`gated_group_rmsnorm` with the gate behind the norm).  Every size and constant is a constructor parameter.
 """
 
 from __future__ import annotations
@@ -63,7 +64,10 @@ class GatedLinearAttention:
 
     def working_bytes(self, step) -> int:
         width = self.n_heads * self.vdim
-        return (self.proj.working_bytes(step, step.rows) + self.decay_down.working_bytes(step, step.rows)
+        chunks = 0
+        if step.sizes is not None and hasattr(step.sizes, "gla_chunk_bytes"):
+            chunks = step.sizes.gla_chunk_bytes(step.seqs, step.rows, step.max_rows_per_seq, self.n_heads, self.dim, self.vdim)
+        return (chunks + self.proj.working_bytes(step, step.rows) + self.decay_down.working_bytes(step, step.rows)
                 + self.decay_up.working_bytes(step, step.rows, out_size=4) + step.matrix(step.rows, width, 4)
                 + step.matrix(step.rows, width, reader=self.out.reader_for_plan(step.act_size))
                 + self.out.working_bytes(step, step.rows, accumulate=True))
@@ -75,7 +79,7 @@ class GatedLinearAttention:
         decays = self.decay_up.forward(ctx, self.decay_down.forward(ctx, x), out_dtype=torch.float32)
         mixed = ctx.new_f32(ctx.n_rows, width)
         k.gla_scan(proj, self.q_off, self.k_off, self.v_off, decays, self.decay_bias, self.tau, self.dim ** -0.5, cache.state,
-                   ctx.seq_start, ctx.seq_slot, mixed, self.n_heads, self.dim, self.vdim)
+                   ctx.seq_start, ctx.seq_slot, mixed, self.n_heads, self.dim, self.vdim, max_rows_per_seq=ctx.max_rows_per_seq)
         gated = ctx.new_activations(ctx.n_rows, width, reader=self.out.reader())
         k.gated_group_rmsnorm(mixed, proj, self.g_off, self.norm_weight, self.norm_eps, gated, self.n_heads, gate_after=True)
         self.out.forward(ctx, gated, out=hidden, accumulate=not fresh)

@@ -534,7 +534,8 @@ class TorchKernels:
         out.copy_(self._clamped_glu(gate_up[:, :ff].double(), gate_up[:, ff:].double(), limit, alpha, shift).to(out.dtype))
 
     # ---- gated linear attention, a norm over a slice, a weighted sum ----
-    def gla_scan(self, proj, q_off, k_off, v_off, z, bias, tau, q_scale, state, seq_start, seq_slot, out, n_heads, dim, vdim):
+    def gla_scan(self, proj, q_off, k_off, v_off, z, bias, tau, q_scale, state, seq_start, seq_slot, out, n_heads, dim, vdim,
+                 max_rows_per_seq=None):
         self.calls.append("gla_scan")
         kw, vw = n_heads * dim, n_heads * vdim
         log_alpha = torch.nn.functional.logsigmoid(z.double() + bias.double()) / tau

@@ -45,10 +45,12 @@ def selector(first, count, width):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("heads,dim,vdim,tau,rank,lengths", [(2, 5, 7, 3.0, 3, [5, 1, 31]), (1, 16, 24, 16.0, 4, [70]), (3, 48, 64, 8.0, 16, [3, 17, 2]),
                                                              (2, 128, 128, 1.0, 8, [40, 9]), (4, 33, 100, 4.0, 5, [1, 1, 1, 1, 1]),
-                                                             (6, 64, 256, 2.0, 2, [130])])
+                                                             (6, 64, 256, 2.0, 2, [130]), (2, 16, 24, 8.0, 4, [700, 64, 1, 333]), (3, 64, 128, 16.0, 8, [1030]),
+                                                             (1, 40, 72, 4.0, 3, [129, 128, 127, 300])])
 def test_gated_linear_attention_scan_norm_and_gate(K, dtype, heads, dim, vdim, tau, rank, lengths):
     """The recurrence over ragged rows of several sequences, into slots in another order than the batch's, then a second step
-    that continues from the states the first one left; behind it the heads' norm with the gate after it."""
+    that continues from the states the first one left; behind it the heads' norm with the gate after it.  The long sequences
+    are walked in chunks side by side (beside short ones that are not), and must come out as if walked in one."""
     rng = np.random.default_rng(heads * dim + vdim)
     kw, vw = heads * dim, heads * vdim
     width = 3 + 2 * kw + 2 * vw + rank
@@ -68,7 +70,7 @@ def test_gated_linear_attention_scan_norm_and_gate(K, dtype, heads, dim, vdim, t
         z = (rows[:, low_off:low_off + rank].astype(np.float64) @ w["m.a2"].T).astype(np.float32)
         mixed = torch.empty(total, vw, device="cuda:0")
         K.gla_scan(dev(rows_t), q_off, k_off, v_off, dev(z), dev(w["m.a2.b"].astype(np.float32)), tau, dim ** -0.5, state, seq_start, seq_slot,
-                   mixed, heads, dim, vdim)
+                   mixed, heads, dim, vdim, max_rows_per_seq=max(lengths))
         out = torch.empty(total, vw, dtype=dtype, device="cuda:0")
         K.gated_group_rmsnorm(mixed, dev(rows_t), g_off, norm_weight, eps, out, heads, gate_after=True)
         for s in range(len(lengths)):
