@@ -831,15 +831,15 @@ def vepelix_config(width, heads, vocab, experts=32, top=4, window=4096, rank=192
     key/value head, a rotation over half a head) beside gated linear attention (keys of 64 and values of 128 a head, decays through
     a rank of 16); `experts` experts of 3/8 of the width of which `top` are used and a shared one of 3/2 of the width in all layers
     but the first, whose feed-forward is dense and three times the width."""
-    stretch = {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}
+    stretch = {"factor": 4.0, "original": 4096, "fast": 16.0, "slow": 1.0}
     mlp = {"kind": "moe", "router": {"experts": experts, "top": top}, "expert": {"ff": 3 * width // 8}, "shared": {"ff": 3 * width // 2}}
     latent = {"type": "latent_attention", "mlp": mlp,
               "mixer": {"heads": heads, "dim": 128, "rot_dim": rot, "vdim": 128, "kv_rank": rank, "q_rank": 3 * width // 8,
-                        "scale": (128 + rot) ** -0.5, "rot": {"base": 500000.0, "dims": rot, "scaling": stretch}}}
+                        "scale": (128 + rot) ** -0.5, "rot": {"base": 10000.0, "dims": rot, "scaling": stretch}}}
     side = {"type": "parallel", "mlp": mlp,
             "mixer": {"left": {"heads": heads, "kv_heads": max(heads // 4, 1), "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
-                               "mask": {"size": window}, "rot": {"base": 1000000.0, "dims": 64, "scaling": stretch}},
-                      "right": {"heads": heads, "dim": 64, "vdim": 128, "tau": 16.0, "decay_rank": 16}, "left_scale": 1.0, "right_scale": 1.0}}
+                               "mask": {"size": window}, "rot": {"base": 100000.0, "dims": 64, "scaling": stretch}},
+                      "right": {"heads": heads, "dim": 64, "vdim": 128, "tau": 8.0, "decay_rank": 16}, "left_scale": 1.0, "right_scale": 1.0}}
     first = dict(latent, mlp={"kind": "dense", "ff": 3 * width, "limit": 7.0})
     return {"architecture": "Vepelix", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "loop": {"start": 1, "stop": 3, "times": 2},
             "layers": [first, latent, side, latent, side, latent]}

@@ -34,7 +34,7 @@ def build_vepelix(config: VepelixConfig):
         config, position_encoding="none", layer_prefix="l{}.", embedding_name="embed", final_norm_name="final.norm",
         head_name="head", final_norm_kind="rmsnorm_zero_centred",
         make_residual=lambda c: StreamsResidual(1, c.hidden),      # one plain residual, in the stream block's form
-        make_pass_input=lambda c: EmbeddingAgain() if c.pass_starts() else None)
+        make_pass_input=lambda c: EmbeddingAgain(c.hidden) if c.pass_starts() else None)
 
 
 register_architecture("Vepelix", VepelixConfig, build_vepelix)

@@ -115,6 +115,9 @@ class EmbeddingAgain:
     graph_safe = True
     graph_safe_rows = None
 
+    def __init__(self, hidden: int):
+        self.hidden = int(hidden)
+
     def tensor_specs(self):
         return []
 
@@ -122,7 +125,7 @@ class EmbeddingAgain:
         pass
 
     def working_bytes(self, step) -> int:
-        return 0      # the copy has the residual's size, which the decoder counts once; this part does not know the width
+        return step.matrix(step.rows, self.hidden, 4)      # the copy of the embedding's output
 
     def keep(self, ctx, hidden):
         return hidden.clone()

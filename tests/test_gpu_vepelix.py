@@ -43,9 +43,9 @@ def selector(first, count, width):
 # ---- kernels alone ------------------------------------------------------------------------------------------
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("heads,dim,vdim,tau,rank,lengths", [(2, 5, 7, 3.0, 3, [5, 1, 31]), (1, 16, 24, 16.0, 4, [70]), (3, 48, 64, 8.0, 16, [3, 17, 2]),
+@pytest.mark.parametrize("heads,dim,vdim,tau,rank,lengths", [(2, 5, 7, 3.0, 3, [5, 1, 31]), (1, 16, 24, 20.0, 4, [70]), (3, 48, 64, 8.0, 16, [3, 17, 2]),
                                                              (2, 128, 128, 1.0, 8, [40, 9]), (4, 33, 100, 4.0, 5, [1, 1, 1, 1, 1]),
-                                                             (6, 64, 256, 2.0, 2, [130]), (2, 16, 24, 8.0, 4, [700, 64, 1, 333]), (3, 64, 128, 16.0, 8, [1030]),
+                                                             (6, 64, 256, 2.0, 2, [130]), (2, 16, 24, 8.0, 4, [700, 64, 1, 333]), (3, 64, 128, 12.0, 8, [1030]),
                                                              (1, 40, 72, 4.0, 3, [129, 128, 127, 300])])
 def test_gated_linear_attention_scan_norm_and_gate(K, dtype, heads, dim, vdim, tau, rank, lengths):
     """The recurrence over ragged rows of several sequences, into slots in another order than the batch's, then a second step
@@ -96,7 +96,7 @@ def attend_plain(q, k, v, scale, window, sinks, first_position):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("heads,kv_heads,hd,past,rows,window", [(8, 2, 64, 0, 2100, 0), (8, 2, 64, 0, 2100, 136), (4, 1, 128, 700, 1, 0), (6, 2, 96, 130, 3, 70),
+@pytest.mark.parametrize("heads,kv_heads,hd,past,rows,window", [(8, 2, 64, 0, 2100, 0), (8, 2, 64, 0, 2100, 150), (4, 1, 128, 700, 1, 0), (6, 2, 96, 130, 3, 70),
                                                                 (2, 1, 256, 5000, 1, 0), (3, 3, 40, 200, 9, 0), (16, 1, 160, 64, 40, 0)])
 def test_a_sink_in_every_attention_kernel(K, dtype, heads, kv_heads, hd, past, rows, window):
     """Prompts of many columns, decode rows, one long context in key splits and head sizes that the matrix cores do not take:
@@ -131,7 +131,7 @@ def test_a_sink_in_every_attention_kernel(K, dtype, heads, kv_heads, hd, past, r
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("heads,kv_heads,dim,vdim,pad,turned,stretch", [(4, 2, 32, 16, 32, 8, None), (2, 1, 96, 192, 192, 96, (8.0, 1024, 32.0, 1.0)),
+@pytest.mark.parametrize("heads,kv_heads,dim,vdim,pad,turned,stretch", [(4, 2, 32, 16, 32, 8, None), (2, 1, 80, 160, 160, 80, (4.0, 512, 16.0, 1.0)),
                                                                         (3, 3, 20, 12, 32, 20, (4.0, 64, 16.0, 1.0)), (1, 1, 64, 64, 64, 0, None)])
 def test_head_norms_and_rotation_in_neighbouring_pairs(K, dtype, heads, kv_heads, dim, vdim, pad, turned, stretch):
     """Queries as the kernel leaves them, and keys and values through the attention that reads them: per-head norms with one
@@ -309,7 +309,7 @@ NO_EXPERTS = {
     "architecture": "Vepelix", "vocab": 83, "width": 64, "norm": {"eps": 1e-5}, "loop": {"start": 0, "stop": 2, "times": 2},
     "layers": [vm.parallel(4, 2, 32, 48, 0.2, 48, 4, 16, 24, 6.0, 8, 1.1, 0.9, dims=16, base=1000.0, stretch=(4.0, 64, 8.0, 1.0), mlp=vm.dense(96, 1.5)),
                vm.latent(4, 16, 16, 32, 48, 24, 0.25, stretch=(8.0, 32, 16.0, 1.0), mlp=vm.dense(40, 3.0)),
-               vm.latent(2, 32, 32, 16, 64, 32, 0.2, base=500000.0)],
+               vm.latent(2, 32, 32, 16, 64, 32, 0.2, base=300000.0)],
 }
 
 
@@ -457,7 +457,7 @@ def test_a_sink_that_outweighs_the_one_key(tmp_path, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("window", [64, 96, 130, 2, 65, 136])
+@pytest.mark.parametrize("window", [64, 96, 130, 2, 65, 141])
 def test_a_key_just_inside_and_just_outside_the_window(tmp_path, dtype, window):
     last = 420
     needle_case(tmp_path, dtype, "window", window, last - window + 1, True)   # the oldest position the window keeps

@@ -101,6 +101,26 @@ def test_the_manifest_is_what_the_configuration_implies(name):
     assert {spec.name: tuple(spec.shape) for spec in model.tensor_specs()} == vm.tensor_shapes(config)
 
 
+def test_the_decays_rank_is_read_from_the_checkpoint_where_the_file_does_not_say_it(tmp_path):
+    config = vm.CONFIGS["mixed"]
+    weights = vm.random_weights(config, 2)
+    silent = copy.deepcopy(config)
+    for layer in silent["layers"]:
+        if layer["type"] == "parallel":
+            layer["mixer"]["right"].pop("decay_rank")
+    folder = vm.write_model(tmp_path / "silent", silent, weights)
+    engine = make_engine(folder)
+    assert engine.model.config.layers[1].mixer.right.decay_rank == 8 and engine.model.config.layers[3].mixer.right.decay_rank == 4
+    tokens = schedules.random_requests(config["vocab"], [33], seed=1)[0]
+    slot = engine.alloc_slot()
+    got = engine.step([StepEntry(slot, tokens, list(range(len(tokens))))]).numpy()
+    assert schedules.relative_error(got, plain.forward(config, weights, tokens)) < 1e-4
+    import io
+    from beholdd import cli
+    out = io.StringIO()
+    assert cli.main(["generate", "--model", folder, "--prompt-ids", "1,2,3", "--max-new-tokens", "4", "--dtype", "bfloat16", "--plan-only"], out=out) == 0
+
+
 def test_a_checkpoint_with_other_tensors_is_refused(tmp_path):
     config = vm.CONFIGS["odd"]
     weights = vm.random_weights(config, 1)

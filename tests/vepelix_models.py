@@ -54,7 +54,7 @@ STRETCH = (4.0, 64, 16.0, 1.0)
 MIXED = {
     "architecture": "Vepelix", "vocab": 97, "width": 64, "norm": {"eps": 1e-5}, "loop": {"start": 1, "stop": 3, "times": 2},
     "layers": [latent(3, 16, 16, 24, 48, 40, 0.3, base=500.0, stretch=STRETCH, mlp=dense(80, 1.2)),
-               parallel(4, 2, 96, 40, 0.12, 70, 2, 16, 24, 8.0, 8, 1.3, 0.8, dims=48, base=1000.0, stretch=(8.0, 128, 32.0, 1.0),
+               parallel(4, 2, 96, 40, 0.12, 70, 2, 16, 24, 8.0, 8, 1.3, 0.8, dims=48, base=1000.0, stretch=(6.0, 128, 20.0, 1.0),
                         mlp=moe(6, 3, 32)),
                latent(2, 24, 8, 16, 56, 24, 0.25, mlp=moe(4, 1, 40, shared=48)),
                parallel(2, 2, 32, 32, 0.2, 0, 3, 8, 8, 2.0, 4, 0.7, 1.1, dims=32, base=100.0)],
@@ -63,7 +63,7 @@ MIXED = {
 # a feed-forward; one expert of which one is used.
 PLAIN = {
     "architecture": "Vepelix", "vocab": 131, "width": 96, "norm": {"eps": 1e-6},
-    "layers": [parallel(1, 1, 64, 64, 0.15, 65, 1, 32, 40, 16.0, 16, 1.0, 1.0, mlp=dense(128, 7.0)),
+    "layers": [parallel(1, 1, 64, 64, 0.15, 65, 1, 32, 40, 12.0, 16, 1.0, 1.0, mlp=dense(128, 7.0)),
                latent(1, 8, 4, 40, 28, 12, 0.6, base=100.0),
                latent(4, 32, 32, 32, 96, 64, 0.2, base=20000.0, stretch=(2.0, 32, 8.0, 2.0), mlp=moe(1, 1, 64, shared=32))],
 }
@@ -78,8 +78,8 @@ ODD = {
 # A loop that runs once and one that is empty in another copy; a cached head of 256 (the matrix-core attention's largest).
 WIDE = {
     "architecture": "Vepelix", "vocab": 211, "width": 128, "norm": {"eps": 1e-6}, "loop": {"start": 1, "stop": 2, "times": 1},
-    "layers": [latent(4, 32, 64, 32, 192, 96, 0.15, base=1e6, stretch=(8.0, 256, 32.0, 1.0), mlp=moe(8, 2, 64, shared=64)),
-               parallel(8, 2, 64, 128, 0.125, 130, 4, 32, 64, 16.0, 16, 1.2, 1.1, dims=64, base=1e6, stretch=(8.0, 256, 32.0, 1.0),
+    "layers": [latent(4, 32, 64, 32, 192, 96, 0.15, base=250000.0, stretch=(16.0, 256, 24.0, 2.0), mlp=moe(8, 2, 64, shared=64)),
+               parallel(8, 2, 64, 128, 0.125, 130, 4, 32, 64, 10.0, 16, 0.9, 1.3, dims=64, base=250000.0, stretch=(16.0, 256, 24.0, 2.0),
                         mlp=moe(8, 2, 64)),
                latent(8, 16, 16, 16, 48, 32, 0.2, mlp=dense(192, 1.5))],
 }
@@ -182,7 +182,7 @@ def drawn_config(seed):
         return moe(experts, int(rng.integers(1, min(experts, 3) + 1)), int(pick(8, 20, 32, 64)), shared=int(pick(0, 16, 40)))
 
     def stretch():
-        return pick(None, (float(pick(2.0, 8.0, 32.0)), int(pick(16, 64, 512)), float(pick(4.0, 32.0)), float(pick(0.5, 1.0))))
+        return pick(None, (float(pick(2.0, 6.0, 32.0)), int(pick(16, 64, 256)), float(pick(4.0, 24.0)), float(pick(0.5, 1.0))))
 
     layers = []
     for _ in range(n_layers):
@@ -190,14 +190,14 @@ def drawn_config(seed):
             rot_dim = int(pick(2, 4, 8, 16, 24))
             layers.append(latent(int(pick(1, 2, 3, 6)), int(pick(4, 8, 20, 32)), rot_dim, int(pick(4, 12, 16, 36)),
                                  int(pick(8, 24, 30, 40, 56, 112)), int(pick(8, 20, 32, 64)), float(pick(0.1, 0.2, 0.35)),
-                                 base=float(pick(100.0, 10000.0, 500000.0)), stretch=stretch(), mlp=feed_forward()))
+                                 base=float(pick(100.0, 10000.0, 300000.0)), stretch=stretch(), mlp=feed_forward()))
         else:
             kv_heads = int(pick(1, 2, 3))
             dim = int(pick(8, 12, 32, 64, 96))
             dims = int(pick(0, *[d for d in (2, 8, 12, 32, 64, 96) if d <= dim]))
             layers.append(parallel(kv_heads * int(pick(1, 2, 4)), kv_heads, dim, int(pick(8, 20, 32, 64, 100)), float(pick(0.1, 0.2, 0.3)),
                                    int(pick(0, 1, 3, 64, 65, 100)), int(pick(1, 2, 5)), int(pick(4, 12, 16, 33, 64)),
-                                   int(pick(4, 10, 16, 40, 72)), float(pick(1.0, 4.0, 16.0)), int(pick(1, 4, 7, 16)),
+                                   int(pick(4, 10, 16, 40, 72)), float(pick(1.0, 4.0, 12.0)), int(pick(1, 4, 7, 16)),
                                    float(pick(0.5, 1.0, 1.2)), float(pick(0.5, 1.0, 1.1)), dims=dims,
                                    base=float(pick(100.0, 10000.0, 1e6)), stretch=stretch() if dims else None, mlp=feed_forward()))
     config = {"architecture": "Vepelix", "vocab": int(pick(37, 64, 150, 301)), "width": width,
