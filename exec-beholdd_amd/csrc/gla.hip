@@ -19,9 +19,9 @@ __device__ inline float log_sigmoid_f32(float x) { return fminf(x, 0.f) - log1pf
 // A workgroup takes a (sequence, head, tile of VT value columns).  Thread (column, slice) keeps rows slice * R .. + R - 1 of its
 // column of S in registers.  GLA_STAGE rows' decays, keys, queries (LDS rows of SL * R floats, zeros beyond dim) and the tile's
 // values are staged at a time; a row's shares of o are added over a wave's slices by lane exchanges and over the waves through
-// LDS, in a fixed order.  The next stage's
-// numbers are asked for (into registers, GLA_AHEAD elements a thread and array; what a stage has beyond that is read when it
-// is staged) before this stage's rows are walked, so that the walk hides their way from memory.
+// LDS, in a fixed order.  The next stage's numbers are asked for (into registers, GLA_AHEAD elements a thread and array; what a
+// stage has beyond that is read when it is staged) before this stage's rows are walked, so that the walk hides their way from
+// memory.
 #define GLA_AHEAD 4
 #define GLA_GROUP 4
 #define GLA_KEPT 8        // key channels a thread keeps a product of decays for: heads of up to 2,048 key dimensions
