@@ -28,4 +28,4 @@ __all__ = ["BLOCKS", "FEED_FORWARDS", "MIXERS", "NORMS", "POSITION_ENCODINGS", "
            "SquaredReLU", "LightningAttention", "LatentAttention", "StreamConnection", "StreamMixingBlock", "StreamsResidual",
            "ScaledLMHead", "LayerNorm", "CappedLMHead", "ScaledEmbedding", "ConvGatedAttention", "StateSpaceScan", "ClampedGLU",
            "RoutedExperts", "LoopInput", "TokenSideInput", "TokenSideTable", "GatedAttention", "MatrixMemory", "PostNormBlock",
-           "GeluTanh"]
+           "GeluTanh", "GatedLinearAttention", "ParallelMixers", "EmbeddingAgain"]
